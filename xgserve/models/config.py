@@ -16,7 +16,7 @@ from typing import Dict, List, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" | "mixtral" | "gpt2" | "dofivik" | "vizonex"
+    arch: str                      # "llama" | "mixtral" | "gpt2" | "dofivik" | "vizonex" | "loluzen"
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -39,6 +39,11 @@ class ModelConfig:
     layer_specs: Optional[List[dict]] = None
     postln_alpha: float = 1.0
     canon_taps: int = 1
+    # "loluzen": factor on the embedding rows, factor on every normed sublayer output, and the run of layers
+    # {"start", "stop", "times"} that is repeated with the same weights (None = every layer once)
+    embed_scale: float = 1.0
+    residual_mult: float = 1.0
+    layer_loop: Optional[dict] = None
 
     @property
     def q_size(self) -> int:
@@ -53,6 +58,8 @@ class ModelConfig:
         if self.layer_specs is not None:
             if self.arch == "vizonex":
                 from .vizonex import count_params
+            elif self.arch == "loluzen":
+                from .loluzen import count_params
             else:
                 from .dofivik import count_params
             return count_params(self)
@@ -66,7 +73,19 @@ class ModelConfig:
         emb = V * H * (1 if self.tie_embeddings else 2)
         return L * (attn + mlp + 2 * H) + emb + H
 
+    def layer_runs(self) -> List[int]:
+        """Indices into layer_specs in the order the layers run (a looped run of layers appears `times` times)."""
+        n = len(self.layer_specs or [])
+        lp = self.layer_loop
+        if not lp:
+            return list(range(n))
+        a, b = int(lp["start"]), int(lp["stop"])
+        return list(range(a)) + list(range(a, b)) * int(lp["times"]) + list(range(b, n))
+
     def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
+        if self.arch == "loluzen":
+            att = [(m.get("left") or m) for m in (self.layer_specs[i]["mixer"] for i in self.layer_runs())]
+            return sum((m["dim"] + m["vdim"]) * m["kv_heads"] * dtype_bytes for m in att)
         if self.arch == "vizonex":
             return sum((m["dim"] + m["vdim"]) * m["kv_heads"] * dtype_bytes
                        for m in (L["mixer"] for L in self.layer_specs if L["type"] == "attention"))
@@ -212,6 +231,77 @@ def _vizonex_tiny_layers():
 
 
 register(vizonex_config("vizonex-tiny", 128, 512, _vizonex_tiny_layers(), taps=3, max_position=1024))
+def loluzen_config(name: str, width: int, vocab: int, layers: List[dict], embed_scale: float = 1.0,
+                   residual_mult: float = 1.0, loop: Optional[dict] = None, eps: float = 1e-5,
+                   max_position: int = 131072) -> ModelConfig:
+    """A Loluzen model: x <- x + m * N(mixer(N(x))), x <- x + m * N(ff(N(x))) with one-plus-weight RMS norms before
+    and after every sublayer; a run of layers may repeat with shared weights (each repetition with a cache of its
+    own, the scaled embedding rows added again before it). Mixers: "attention" (short convolution on q / k / v,
+    per-head q / k norm, partial rotation with rescaled frequencies, per-head output gate) and "parallel" (a biased
+    attention branch with a logarithmic distance penalty and post-softmax head mixing beside a gated linear
+    recurrence whose forget gate also sets the write strength). Feed-forward: dense squared-relu with biases, or none."""
+    def need(d, keys, where):
+        for k in keys:
+            if k not in d:
+                raise ValueError(f"{where}: missing {k!r}")
+
+    def gqa(m, w):
+        need(m, ("heads", "kv_heads", "dim", "vdim", "scale"), w)
+        if m["heads"] < 1 or m["kv_heads"] < 1 or m["heads"] % m["kv_heads"]:
+            raise ValueError(f"{w}: heads must be a positive multiple of kv_heads")
+    if not layers:
+        raise ValueError("a model needs at least one layer")
+    for i, L in enumerate(layers):
+        m, w = L.get("mixer") or {}, f"layer {i}"
+        if L.get("type") == "attention":
+            gqa(m, w)
+            if not 1 <= int(m.get("conv", 1)) <= 8:
+                raise ValueError(f"{w}: conv must be in [1, 8]")
+            rot = m.get("rot")
+            if rot is not None:
+                need(rot, ("base", "dims"), w)
+                if rot["dims"] % 2 or not 0 <= rot["dims"] <= m["dim"]:
+                    raise ValueError(f"{w}: rot.dims must be even and at most dim")
+                if rot.get("scaling") is not None:
+                    need(rot["scaling"], ("factor", "low", "high", "original"), w)
+        elif L.get("type") == "parallel":
+            need(m, ("left", "right"), w)
+            gqa(m["left"], w + " left")
+            need(m["right"], ("heads", "dim", "vdim"), w + " right")
+            if m["right"]["dim"] > 256:
+                raise ValueError(f"{w}: recurrent head sizes above 256 are not supported")
+        else:
+            raise ValueError(f"{w}: unknown mixer type {L.get('type')!r}")
+        mlp = L.get("mlp")
+        if mlp is not None:
+            if mlp.get("kind") != "dense":
+                raise ValueError(f"{w}: unknown feed-forward kind {mlp.get('kind')!r}")
+            need(mlp, ("ff",), w)
+    if loop is not None:
+        need(loop, ("start", "stop", "times"), "loop")
+        if not (0 <= loop["start"] < loop["stop"] <= len(layers)) or loop["times"] < 1:
+            raise ValueError("loop: needs 0 <= start < stop <= number of layers and times >= 1")
+    att = [(L["mixer"].get("left") or L["mixer"]) for L in layers]
+    heads = max(m["heads"] for m in att)
+    hd = max(max(m["dim"], m["vdim"]) for m in att)
+    ff = max([L["mlp"]["ff"] for L in layers if L.get("mlp")] or [0])
+    return ModelConfig(name, "loluzen", width, len(layers), heads, max(m["kv_heads"] for m in att), hd, ff, vocab,
+                       max_position, 0.0, None, eps, False, bos_token_id=0, eos_token_ids=[], layer_specs=layers,
+                       embed_scale=float(embed_scale), residual_mult=float(residual_mult), layer_loop=loop)
+
+
+def _loluzen_tiny_layers():
+    att = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.2, "conv": 4,
+           "rot": {"base": 10000.0, "dims": 16, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}}}
+    par = {"left": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.25},
+           "right": {"heads": 2, "dim": 16, "vdim": 32}}
+    return [{"type": "parallel", "mixer": par, "mlp": {"kind": "dense", "ff": 192}},
+            {"type": "attention", "mixer": att, "mlp": None},
+            {"type": "attention", "mixer": dict(att), "mlp": {"kind": "dense", "ff": 160}}]
+
+
+register(loluzen_config("loluzen-tiny", 128, 512, _loluzen_tiny_layers(), embed_scale=4.0, residual_mult=0.5,
+                        loop={"start": 1, "stop": 2, "times": 2}, max_position=1024))
 register(ModelConfig("gpt2-tiny", "gpt2", 128, 2, 2, 2, 64, 512, 512, 256, 0.0, tie_embeddings=True,
                      bos_token_id=0, eos_token_ids=[0], dtype="float32"))
 
@@ -237,6 +327,9 @@ def from_hf_config(path: str, name: Optional[str] = None) -> ModelConfig:
     if c.get("architecture") == "Vizonex":
         return vizonex_config(name or "vizonex", c["width"], c["vocab"], c["layers"], c["canon"]["taps"],
                               c["norm"]["eps"], int(c["max_positions"]))
+    if c.get("architecture") == "Loluzen":
+        return loluzen_config(name or "loluzen", c["width"], c["vocab"], c["layers"], c["embedding"]["scale"],
+                              c["residual_mult"], c.get("loop"), c["norm"]["eps"], int(c.get("max_position", 131072)))
     mt = c.get("model_type", "llama")
     eos = c.get("eos_token_id", 2)
     eos = eos if isinstance(eos, list) else [eos]

@@ -22,15 +22,24 @@ from .config import ModelConfig, get_config
 from .dofivik import DofivikForCausalLM
 from .gpt2 import GPT2ForCausalLM
 from .llama import LlamaForCausalLM
+from .loluzen import LoluzenForCausalLM
 from .vizonex import VizonexForCausalLM
 
 
 def model_class(cfg: ModelConfig):
-    return {"gpt2": GPT2ForCausalLM, "dofivik": DofivikForCausalLM, "vizonex": VizonexForCausalLM}.get(cfg.arch, LlamaForCausalLM)
+    return {"gpt2": GPT2ForCausalLM, "dofivik": DofivikForCausalLM, "vizonex": VizonexForCausalLM,
+            "loluzen": LoluzenForCausalLM}.get(cfg.arch, LlamaForCausalLM)
 
 
 def _resolve_shapes(cfg: ModelConfig, checkpoint: str) -> None:
-    """Sizes that only a tensor's shape gives (Dofivik: the rank of the decay projection)."""
+    """Sizes that only a tensor's shape gives (Dofivik: the rank of the decay projection; Loluzen: the taps of
+    a short convolution when the configuration leaves them out)."""
+    if cfg.arch == "loluzen":
+        r = _Reader(checkpoint)
+        for i, spec in enumerate(cfg.layer_specs):
+            if spec["type"] == "attention" and "conv" not in spec["mixer"]:
+                spec["mixer"]["conv"] = int(r.shape(f"l{i}.mix.q.conv")[1]) if r.has(f"l{i}.mix.q.conv") else 1
+        return
     if cfg.arch != "dofivik":
         return
     r = _Reader(checkpoint)
@@ -123,6 +132,8 @@ def load_checkpoint(model, path: str) -> None:
         _load_dofivik(model, r)
     elif cfg.arch == "vizonex":
         _load_vizonex(model, r)
+    elif cfg.arch == "loluzen":
+        _load_loluzen(model, r)
     else:
         _load_llama(model, r)
 
@@ -281,6 +292,66 @@ def _load_vizonex(m, r: _Reader):
         dst.copy_(src.to(dst.dtype))
 
 
+def _loluzen_tensors(m):
+    """(checkpoint name, parameter, index of a fused parameter or None) for every tensor."""
+    out = [("embed", m.embed, None), ("head", m.head, None), ("final.norm", m.final_norm, None)]
+    for i, L in enumerate(m.layers):
+        b, x = f"l{i}.", L.mix
+        out += [(b + "norm1", L.norm1, None), (b + "norm1b", L.norm1b, None)]
+        if L.kind == "attention":
+            nq, nk, nv = x.nq, x.nk, x.nv
+            out += [(b + "mix.q", x.in_proj, slice(0, nq)), (b + "mix.k", x.in_proj, slice(nq, nq + nk)),
+                    (b + "mix.v", x.in_proj, slice(nq + nk, x.ch)), (b + "mix.g", x.in_proj, slice(x.ch, x.ch + x.H)),
+                    (b + "mix.q.conv", x.conv_w, slice(0, nq)), (b + "mix.k.conv", x.conv_w, slice(nq, nq + nk)),
+                    (b + "mix.v.conv", x.conv_w, slice(nq + nk, x.ch)), (b + "mix.q.norm", x.q_norm, None),
+                    (b + "mix.k.norm", x.k_norm, None), (b + "mix.o", x.o, None)]
+        else:
+            a, r = x.left, x.right
+            at = 0
+            for name, rows, bias in (("left.q", a.nq, True), ("left.k", a.nk, True), ("left.v", a.nv, True),
+                                     ("left.g", a.H, False), ("right.q", r.n, False), ("right.f", r.n, True),
+                                     ("right.v", r.H * r.dv, False)):
+                out.append((b + "mix." + name, x.in_proj, slice(at, at + rows)))
+                if bias:
+                    out.append((b + "mix." + name + ".b", x.in_bias, slice(at, at + rows)))
+                at += rows
+            out += [(b + "mix.left.r1", a.r1, None), (b + "mix.left.r2", a.r2, None), (b + "mix.left.talk", a.talk, None),
+                    (b + "mix.left.o", a.o, None), (b + "mix.left.out", a.out_norm, None),
+                    (b + "mix.right.lower", r.lower, None), (b + "mix.right.norm", r.norm, None),
+                    (b + "mix.right.o", r.o, None), (b + "mix.right.out", r.out_norm, None)]
+        if L.mlp is not None:
+            out += [(b + "norm2", L.norm2, None), (b + "norm2b", L.norm2b, None), (b + "mlp.up", L.mlp.up, None),
+                    (b + "mlp.up.b", L.mlp.up_b, None), (b + "mlp.down", L.mlp.down, None),
+                    (b + "mlp.down.b", L.mlp.down_b, None)]
+    return out
+
+
+def _load_loluzen(m, r: _Reader):
+    """Tensors `embed`, `head`, `final.norm`, `l<i>.<norm1|norm1b|norm2|norm2b>`, `l<i>.mix.*`, `l<i>.mlp.*`
+    ([out, in] matrices). The projections that read the same input (and their biases) are fused row-wise on load."""
+    for name, p, idx in _loluzen_tensors(m):
+        src = r.get(name)
+        dst = p.data if idx is None else p.data[idx]
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"shape mismatch for {name}: model {tuple(dst.shape)} vs checkpoint {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+
+def _save_loluzen(model, path: str) -> None:
+    from safetensors.torch import save_file
+    cfg = model.cfg
+    t = {}
+    for name, p, idx in _loluzen_tensors(model):
+        v = p.data if idx is None else p.data[idx]
+        t[name] = v.detach().to(torch.bfloat16).contiguous().cpu()
+    save_file(t, os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump({"architecture": "Loluzen", "width": cfg.hidden_size, "vocab": cfg.vocab_size,
+                   "embedding": {"scale": cfg.embed_scale}, "residual_mult": cfg.residual_mult,
+                   "layers": cfg.layer_specs, "loop": cfg.layer_loop, "norm": {"eps": cfg.norm_eps},
+                   "max_position": cfg.max_position}, f, indent=1)
+
+
 def _save_vizonex(model, path: str) -> None:
     from safetensors.torch import save_file
     cfg = model.cfg
@@ -324,6 +395,8 @@ def save_checkpoint(model, path: str) -> None:
         return _save_dofivik(model, path)
     if cfg.arch == "vizonex":
         return _save_vizonex(model, path)
+    if cfg.arch == "loluzen":
+        return _save_loluzen(model, path)
     t: Dict[str, torch.Tensor] = {}
     if cfg.arch == "gpt2":
         t["transformer.wte.weight"] = model.wte

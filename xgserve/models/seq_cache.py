@@ -26,6 +26,7 @@ class LayerCache:
     delta: Optional[torch.Tensor] = None    # delta rule: [slots, heads, dim, dim]
     mix_conv: Optional[torch.Tensor] = None  # a mixer's own short convolution: [slots, taps - 1, channels]
     ssm: Optional[torch.Tensor] = None      # state-space recurrence: [slots, heads, state, vdim]
+    gla: Optional[torch.Tensor] = None      # gated linear recurrence: [slots, heads, dim, vdim]
 
 
 @dataclass

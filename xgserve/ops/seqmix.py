@@ -46,13 +46,13 @@ def _i32(t: torch.Tensor) -> torch.Tensor:
 
 # ---------------------------------------------------------------------------- embedding
 def embed_rows(ids: torch.Tensor, table: torch.Tensor, pos_table: Optional[torch.Tensor] = None,
-               positions: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """fp32 rows table[ids] (zero rows for ids outside the table); with `pos_table` the learned vector
+               positions: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """fp32 rows table[ids] * scale (zero rows for ids outside the table); with `pos_table` the learned vector
     pos_table[positions] is added (unscaled)."""
     V, W = table.shape
     if not native_device(table):
         ok = (ids >= 0) & (ids < V)
-        out = table[ids.long().clamp(0, V - 1)].float()
+        out = table[ids.long().clamp(0, V - 1)].float() * scale
         out[~ok] = 0
         if pos_table is not None:
             pk = (positions >= 0) & (positions < pos_table.shape[0])
@@ -65,7 +65,7 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor, pos_table: Optional[torch
         assert pos_table.dtype == table.dtype and pos_table.shape[1] == W and pos_table.is_contiguous()
     mixers().embed_rows(_i32(ids).data_ptr(), table.data_ptr(), is_f32(table), out.data_ptr(), ids.shape[0], W, V,
                         _p(pos_table), _i32(positions).data_ptr() if pos_table is not None else 0,
-                        pos_table.shape[0] if pos_table is not None else 0, stream_ptr())
+                        pos_table.shape[0] if pos_table is not None else 0, float(scale), stream_ptr())
     return out
 
 
@@ -173,10 +173,24 @@ def scaled_add_rmsnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tens
 
 
 # ---------------------------------------------------------------------------- rotation table
-def build_rot_table(dims: int, base: float, max_pos: int, device="cpu") -> torch.Tensor:
-    """fp32 [max_pos, dims / 2, 2] = (cos, sin) of position * base^(-2 i / dims): the angles of the
-    interleaved-pair rotation (dimension 2i with 2i + 1), evaluated in fp64."""
+def rot_frequencies(dims: int, base: float, scaling: Optional[dict] = None) -> torch.Tensor:
+    """fp64 [dims / 2]: f_i = base^(-2 i / dims); with `scaling` {factor, low, high, original} each frequency is
+    rescaled by its wavelength l = 2 pi / f: kept where l < original / high, divided by factor where
+    l > original / low, and in between blended, (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
     inv = base ** (-torch.arange(0, dims, 2, dtype=torch.float64) / dims)
+    if scaling is None:
+        return inv
+    factor, low, high, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+    wave = 2.0 * math.pi / inv
+    s = ((orig / wave - low) / (high - low)) if high != low else torch.ones_like(inv)
+    mid = (1.0 - s) * inv / factor + s * inv
+    return torch.where(wave < orig / high, inv, torch.where(wave > orig / low, inv / factor, mid))
+
+
+def build_rot_table(dims: int, base: float, max_pos: int, device="cpu", scaling: Optional[dict] = None) -> torch.Tensor:
+    """fp32 [max_pos, dims / 2, 2] = (cos, sin) of position * f_i (rot_frequencies): the angles of the
+    interleaved-pair rotation (dimension 2i with 2i + 1), evaluated in fp64."""
+    inv = rot_frequencies(dims, base, scaling)
     ang = torch.outer(torch.arange(max_pos, dtype=torch.float64), inv)
     return torch.stack([ang.cos(), ang.sin()], -1).float().contiguous().to(device)
 
@@ -460,21 +474,34 @@ def qk_norm_cache(proj: torch.Tensor, nq: int, nk: int, nv: int, wq: Optional[to
     return q
 
 
+V_OWN, V_ALL = -1, -2   # masked_attention(values=...): the query head's own key/value head, or every head's values
+V_ALL_MAX = 256         # ... V_ALL serves up to this many value columns (G * dv) per query head
+
+
 def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, H: int, G: int, dk: int, dv: int,
                      mask: int, size: int, scale: float, temp: Optional[torch.Tensor], sink: Optional[torch.Tensor],
-                     block_size: int, sm: SeqMeta) -> torch.Tensor:
+                     block_size: int, sm: SeqMeta, gate: Optional[torch.Tensor] = None,
+                     dist: Optional[tuple] = None, values: int = V_OWN) -> torch.Tensor:
     """Softmax attention of H query heads over G cached key/value heads (query head h reads head h // (H / G)).
-    A query at position i sees keys first_visible(mask, size, i) .. i of its own sequence; positions do not
-    enter the scores. score = (q . k) * scale * temp[h]; with `sink` the denominator also holds exp(sink[h]),
-    a term with no key and no value. q [T, H * dk]; caches [rows, G * dk] / [rows, G * dv]; returns [T, H * dv]."""
+    A query at position i sees keys first_visible(mask, size, i) .. i of its own sequence. score = (q . k) * scale
+    * temp[h]; with `dist` = (r1, r2) (fp32 [H] each) the score of key j loses r1[h] * ln(1 + r2[h] * (i - j)),
+    otherwise positions do not enter the scores; with `sink` the denominator also holds exp(sink[h]), a term with no
+    key and no value; with `gate` ([T, >= H], row-strided) head h's output is multiplied by sigmoid(gate[t, h]).
+    `values`: V_OWN: head h weighs the values of its own key/value head, returns [T, H * dv]; V_ALL: the values of
+    all G heads side by side, returns [T, H * G * dv] (what mixing of the heads' weight maps needs);
+    c >= 0: the values of head c for every query head.
+    q [T, H * dk]; caches [rows, G * dk] / [rows, G * dv]."""
     T = q.shape[0]
-    out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    dvo = G * dv if values == V_ALL else dv           # value columns per query head
+    out = torch.empty(T, H * dvo, dtype=q.dtype, device=q.device)
     if native_device(q):
         assert q.is_contiguous() and kcache.is_contiguous() and vcache.is_contiguous()
-        assert kcache.dtype == vcache.dtype == q.dtype
+        assert kcache.dtype == vcache.dtype == q.dtype and -2 <= values < G
+        assert gate is None or (gate.stride(1) == 1 and gate.dtype == q.dtype and gate.shape[1] >= H)
+        r1, r2 = dist if dist is not None else (None, None)
         bt = _i32(sm.block_tables)
         single = sm.max_q == 1 and T == sm.num_seqs
-        if ATTN_MFMA and q.dtype == torch.bfloat16 and dk % 32 == 0 and dv % 16 == 0 and dk <= 128 and dv <= 128 \
+        if ATTN_MFMA and q.dtype == torch.bfloat16 and dk % 32 == 0 and dv % 16 == 0 and dk <= 128 and dvo <= 256 \
                 and (not single or H // G <= 64):
             # matrix cores: prompt portions (also beside single tokens) as 16 tokens x one head per wave, steps of
             # single tokens as the query heads of one key/value head per wave
@@ -483,17 +510,19 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
                 tiles = (size + 63) // 64 if mask != MASK_CAUSAL else ATTN_MAX_SPLITS
                 nsplit = max(1, min(ATTN_MAX_SPLITS, tiles, ATTN_SPLIT_WGS // max(1, T * G)))
                 if nsplit > 1:
-                    part_o = torch.empty(nsplit * T * H * dv, dtype=torch.float32, device=q.device)
+                    part_o = torch.empty(nsplit * T * H * dvo, dtype=torch.float32, device=q.device)
                     part_ml = torch.empty(nsplit * T * H * 2, dtype=torch.float32, device=q.device)
             mixers().masked_attention_mfma(q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(), bt.shape[1],
                                            block_size, _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
                                            _i32(sm.slots).data_ptr(), _p(temp), _p(sink), out.data_ptr(), T, sm.num_seqs,
                                            sm.max_q, H, G, dk, dv, int(mask), int(size), float(scale), nsplit,
-                                           _p(part_o), _p(part_ml), stream_ptr())
+                                           _p(part_o), _p(part_ml), _p(gate), gate.stride(0) if gate is not None else 0,
+                                           _p(r1), _p(r2), int(values), stream_ptr())
             return out
         mixers().masked_attention(q.data_ptr(), is_f32(q), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(),
                                   bt.shape[1], block_size, _i32(sm.positions).data_ptr(), _i32(sm.token_seq).data_ptr(),
                                   _p(temp), _p(sink), out.data_ptr(), T, H, G, dk, dv, int(mask), int(size), float(scale),
+                                  _p(gate), gate.stride(0) if gate is not None else 0, _p(r1), _p(r2), int(values),
                                   stream_ptr())
         return out
     kr, vr = kcache.view(-1, G, dk), vcache.view(-1, G, dv)
@@ -509,12 +538,21 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         keys = torch.arange(first_visible(mask, size, pos[t]), pos[t] + 1)
         idx = sm.block_tables[s][(keys // block_size).long()].long() * block_size + keys % block_size
         kk = kr[idx].float().repeat_interleave(rep, 1)   # [n, H, dk]
-        vv = vr[idx].float().repeat_interleave(rep, 1)
         sc = torch.einsum("hd,nhd->hn", qf[t], kk) * (scale * tmp)[:, None]
+        if dist is not None:
+            sc = sc - dist[0][:, None] * torch.log1p(dist[1][:, None] * (pos[t] - keys).float()[None, :])
         if sink is not None:
             sc = torch.cat([sc, sink[:, None]], 1)
         p = torch.softmax(sc, -1)[:, :keys.numel()]
-        out[t] = torch.einsum("hn,nhd->hd", p, vv).reshape(H * dv).to(out.dtype)
+        if values == V_ALL:
+            o = torch.einsum("hn,nd->hd", p, vr[idx].float().reshape(keys.numel(), G * dv))
+        elif values >= 0:
+            o = torch.einsum("hn,nd->hd", p, vr[idx][:, values].float())
+        else:
+            o = torch.einsum("hn,nhd->hd", p, vr[idx].float().repeat_interleave(rep, 1))
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t, :H].float())[:, None]
+        out[t] = o.reshape(H * dvo).to(out.dtype)
     return out
 
 
@@ -553,20 +591,26 @@ def ssm_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A_l
     return y
 
 
-def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, eps: float, groups: int,
+def gated_group_norm(y: torch.Tensor, z: Optional[torch.Tensor], w: torch.Tensor, eps: float, groups: int,
                      out_dtype: torch.dtype) -> torch.Tensor:
-    """v = y * silu(z); each of `groups` equal parts of a row divided by its own root mean square; times w.
-    y fp32 [T, n]; z [T, n] (row-strided activation)."""
+    """v = y * silu(z) (v = y when z is None); each of `groups` equal parts of a row divided by its own root mean
+    square; times w, which holds one weight per column or one period of a repeating pattern (e.g. a weight of one
+    head's size shared by all heads). y fp32 [T, n]; z [T, n] (row-strided activation)."""
     T, n = y.shape
+    assert n % groups == 0 and n % w.numel() == 0
     if not native_device(y):
-        zf = z.float()
-        v = (y * zf * torch.sigmoid(zf)).view(T, groups, n // groups)
+        v = y
+        if z is not None:
+            zf = z.float()
+            v = y * zf * torch.sigmoid(zf)
+        v = v.view(T, groups, n // groups)
         v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, n)
-        return (v * w).to(out_dtype)
+        return (v * w.repeat(n // w.numel())).to(out_dtype)
     out = torch.empty(T, n, dtype=out_dtype, device=y.device)
-    assert y.is_contiguous() and z.stride(1) == 1 and z.dtype == out_dtype
-    mixers().gated_group_norm(y.data_ptr(), z.data_ptr(), is_f32(z), z.stride(0), w.data_ptr(), float(eps),
-                              out.data_ptr(), T, n, groups, stream_ptr())
+    assert y.is_contiguous() and y.dtype == torch.float32 and w.dtype == torch.float32
+    assert z is None or (z.stride(1) == 1 and z.dtype == out_dtype)
+    mixers().gated_group_norm(y.data_ptr(), _p(z), is_f32(out), z.stride(0) if z is not None else 0, w.data_ptr(),
+                              w.numel(), float(eps), out.data_ptr(), T, n, groups, stream_ptr())
     return out
 
 
@@ -662,4 +706,173 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
                    False, y.data_ptr(), 0, 0.0, 0.0, MOE_MFMA, stream_ptr())
     out = torch.empty(T, W, dtype=torch.float32, device=dev)
     M.moe_combine(y.data_ptr(), dest.data_ptr(), wts.data_ptr(), T, top, W, out.data_ptr(), stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- norm before and after a sublayer
+def post_norm_residual(x: torch.Tensor, y: Optional[torch.Tensor], y_bias: Optional[torch.Tensor],
+                       post_w: Optional[torch.Tensor], mult: float, extra: Optional[torch.Tensor],
+                       next_w: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype] = None,
+                       w_offset: float = 1.0, y2: Optional[torch.Tensor] = None,
+                       pre_w: Optional[tuple] = None) -> Optional[torch.Tensor]:
+    """A sublayer's output is normed before it joins the residual, and the next sublayer's input norm follows:
+        u  = y + y_bias                                    (pre_w is None)
+        u  = (N0(y) * pre_w[0] + N0(y2) * pre_w[1]) / 2    (two branches, each normed with a plain weight first)
+        x <- x + mult * N0(u) * (w_offset + post_w) + extra
+        n  = N0(x) * (w_offset + next_w)
+    with N0(v) = v / sqrt(mean(v^2) + eps). x fp32 [T, W] is updated in place; y / y2 activation tensors or fp32,
+    row-strided; y_bias, the weights fp32 [W]; extra fp32 [T, W]. y None: only `extra` is added. Returns n as
+    `out_dtype` (None when next_w is None)."""
+    T, W = x.shape
+
+    def n0(v):
+        return v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    if not native_device(x):
+        if y is not None:
+            u = y.float()
+            if pre_w is not None:
+                u = 0.5 * (n0(u) * pre_w[0] + n0(y2.float()) * pre_w[1])
+            elif y_bias is not None:
+                u = u + y_bias
+            x.add_(mult * n0(u) * (w_offset + post_w))
+        if extra is not None:
+            x.add_(extra)
+        return None if next_w is None else (n0(x) * (w_offset + next_w)).to(out_dtype)
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    for t in (y, y2):
+        assert t is None or (t.stride(1) == 1 and t.shape == x.shape)
+    assert (pre_w is None) == (y2 is None) and (y2 is None or y2.dtype == y.dtype)
+    assert extra is None or (extra.dtype == torch.float32 and extra.is_contiguous() and extra.shape == x.shape)
+    out = torch.empty(T, W, dtype=out_dtype, device=x.device) if next_w is not None else None
+    mixers().post_norm_residual(x.data_ptr(), _p(y), is_f32(y) if y is not None else True,
+                                y.stride(0) if y is not None else 0, _p(y_bias), _p(y2),
+                                y2.stride(0) if y2 is not None else 0, _p(pre_w[0]) if pre_w else 0,
+                                _p(pre_w[1]) if pre_w else 0, _p(post_w), float(mult), _p(extra), _p(next_w),
+                                float(w_offset), float(eps), _p(out), is_f32(out) if out is not None else True, T, W,
+                                stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- per-head q / k norm, rotation, cache append
+def head_norm_rope_cache(src: torch.Tensor, H: int, G: int, dk: int, dv: int, wq: Optional[torch.Tensor],
+                         wk: Optional[torch.Tensor], eps: float, rot: Optional[torch.Tensor], rot_dims: int, sm: SeqMeta,
+                         kcache: torch.Tensor, vcache: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """From rows [q (H dk) | k (G dk) | v (G dv)] (fp32 or an activation tensor, row-strided): every q head and
+    every k head is RMS-normed over its own dk entries with one weight of size dk shared by the heads (wq / wk, None
+    = no norm), then the first rot_dims entries of each head are rotated pairwise (entry 2i with 2i + 1) by the
+    table row of the token's position (rot fp32 [positions, rot_dims / 2, 2], None = no rotation). q is returned
+    [T, H dk]; k and v go to cache rows slot_mapping[t]."""
+    T = src.shape[0]
+    nq, nk, nv = H * dk, G * dk, G * dv
+    q = torch.empty(T, nq, dtype=out_dtype, device=src.device)
+    if native_device(src):
+        assert src.stride(1) == 1 and kcache.is_contiguous() and vcache.is_contiguous()
+        assert kcache.dtype == vcache.dtype == out_dtype and kcache.shape[-1] == nk and vcache.shape[-1] == nv
+        assert rot is None or (rot.dtype == torch.float32 and rot.is_contiguous() and rot.shape[1] * 2 == rot_dims)
+        assert rot_dims % 2 == 0 and rot_dims <= dk
+        mixers().head_norm_rope_cache(src.data_ptr(), is_f32(src), src.stride(0), H, G, dk, dv, _p(wq), _p(wk),
+                                      float(eps), _p(rot), rot.shape[0] if rot is not None else 0,
+                                      rot_dims if rot is not None else 0, _i32(sm.positions).data_ptr(),
+                                      _i32(sm.slot_mapping).data_ptr(), q.data_ptr(), kcache.data_ptr(),
+                                      vcache.data_ptr(), is_f32(q), T, stream_ptr())
+        return q
+    pf = src.float()
+
+    def prep(v, n, w):
+        v = v.reshape(T, n, dk)
+        if w is not None:
+            v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w
+        if rot is not None and rot_dims:
+            v = _rotate_pairs(v, rot, sm.positions, rot_dims)
+        return v.reshape(T, n * dk)
+    q.copy_(prep(pf[:, :nq], H, wq).to(out_dtype))
+    ok = sm.slot_mapping >= 0
+    rows = sm.slot_mapping[ok].long()
+    kcache.view(-1, nk)[rows] = prep(pf[:, nq:nq + nk], G, wk)[ok].to(kcache.dtype)
+    vcache.view(-1, nv)[rows] = pf[:, nq + nk:nq + nk + nv][ok].to(vcache.dtype)
+    return q
+
+
+# ---------------------------------------------------------------------------- mixing the heads' weight maps
+def talk_mix(o_all: torch.Tensor, talk: torch.Tensor, H: int, G: int, dv: int,
+             gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Softmax weights mixed over heads AFTER the softmax, p'_h = sum_g talk[h, g] p_g, applied to the values of head
+    h's own key/value head c(h) = h // (H / G), equal  sum_g talk[h, g] * (p_g V_c(h)). o_all [T, H * G * dv] holds
+    p_g V_c for every (g, c) (masked_attention with values=V_ALL); returns [T, H * dv], head h's row times
+    sigmoid(gate[t, h]) when `gate` ([T, >= H], row-strided) is given. The sum over g is fp32."""
+    T = o_all.shape[0]
+    if not native_device(o_all):
+        o = o_all.float().view(T, H, G, dv)
+        sel = o[:, :, torch.arange(H) // (H // G), :]            # [T, g, h, dv]: head g's weights on h's values
+        out = torch.einsum("hg,tghd->thd", talk.float(), sel)
+        if gate is not None:
+            out = out * torch.sigmoid(gate[:, :H].float())[:, :, None]
+        return out.reshape(T, H * dv).to(o_all.dtype)
+    assert o_all.is_contiguous() and talk.dtype == torch.float32 and talk.is_contiguous() and talk.shape == (H, H)
+    assert gate is None or (gate.stride(1) == 1 and gate.dtype == o_all.dtype)
+    out = torch.empty(T, H * dv, dtype=o_all.dtype, device=o_all.device)
+    mixers().talk_mix(o_all.data_ptr(), is_f32(o_all), talk.data_ptr(), _p(gate), gate.stride(0) if gate is not None else 0,
+                      out.data_ptr(), T, H, G, dv, stream_ptr())
+    return out
+
+
+# ---------------------------------------------------------------------------- gated linear recurrence
+def lower_bound_gates(proj: torch.Tensor, off_q: int, off_f: int, n: int, f_bias: Optional[torch.Tensor],
+                      lower: torch.Tensor):
+    """From a fused projection row: q = silu(proj[off_q : off_q + n]) and the forget gate
+    f = l + (1 - l) * sigmoid(proj[off_f : off_f + n] + f_bias), bounded below by l = `lower` (fp32 [n]).
+    Returns (q, f), fp32 [T, n] each."""
+    T = proj.shape[0]
+    if not native_device(proj):
+        pf = proj.float()
+        z = pf[:, off_q:off_q + n]
+        g = pf[:, off_f:off_f + n] + (f_bias if f_bias is not None else 0.0)
+        return z * torch.sigmoid(z), lower + (1.0 - lower) * torch.sigmoid(g)
+    assert proj.stride(1) == 1 and lower.dtype == torch.float32
+    qf = torch.empty(2, T, n, dtype=torch.float32, device=proj.device)
+    mixers().lower_bound_gates(proj.data_ptr(), is_f32(proj), proj.stride(0), off_q, off_f, n, _p(f_bias),
+                               lower.data_ptr(), qf[0].data_ptr(), qf[1].data_ptr(), T, stream_ptr())
+    return qf[0], qf[1]
+
+
+def gated_linear_scan(q: torch.Tensor, f: torch.Tensor, k: Optional[torch.Tensor], v: torch.Tensor, state: torch.Tensor,
+                      H: int, dk: int, dv: int, sm: SeqMeta) -> torch.Tensor:
+    """Per head a [dk x dv] fp32 state with one decay per row:  S <- diag(f) S + k v^T,  o = S^T q;  k = 1 - f when
+    `k` is None (the forget gate also decides what is written). q, f, k fp32 [T, H dk]; v [T, H dv] (row-strided
+    activation). state fp32 [slots, H, dk, dv] is carried and updated. Returns o fp32 [T, H dv]."""
+    T = q.shape[0]
+    o = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+    if native_device(q):
+        assert q.dtype == f.dtype == torch.float32 and q.is_contiguous() and f.is_contiguous() and v.stride(1) == 1
+        assert k is None or (k.dtype == torch.float32 and k.is_contiguous())
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dk, dv)
+        mixers().gated_linear_scan(q.data_ptr(), f.data_ptr(), _p(k), v.data_ptr(), is_f32(v), v.stride(0),
+                                   state.data_ptr(), _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
+                                   _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, dk, dv, stream_ptr())
+        return o
+    qh, fh = q.view(T, H, dk), f.view(T, H, dk)
+    kh = (1.0 - fh) if k is None else k.view(T, H, dk)
+    vh = v.float().reshape(T, H, dv)
+    qsl, sl, slots = sm.qsl.tolist(), sm.seq_lens.tolist(), sm.slots.tolist()
+    for s in range(sm.num_seqs):
+        lo, hi = qsl[s], qsl[s + 1]
+        if slots[s] < 0 or hi <= lo:
+            continue
+        S = state[slots[s]].clone() if sl[s] - (hi - lo) > 0 else torch.zeros(H, dk, dv)
+        for t in range(lo, hi):
+            S = fh[t][:, :, None] * S + kh[t][:, :, None] * vh[t][:, None, :]
+            o[t] = torch.einsum("hkd,hk->hd", S, qh[t]).reshape(H * dv)
+        state[slots[s]] = S
+    return o
+
+
+# ---------------------------------------------------------------------------- squared relu
+def relu2(z: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """max(z + bias, 0)^2 (bias fp32 per column)."""
+    if not native_device(z):
+        v = z.float() + (bias if bias is not None else 0)
+        return torch.relu(v).pow(2).to(z.dtype)
+    assert z.is_contiguous()
+    out = torch.empty_like(z)
+    mixers().relu2(z.data_ptr(), is_f32(z), _p(bias), out.data_ptr(), z.numel(), z.shape[-1], stream_ptr())
     return out
