@@ -9,8 +9,17 @@
 //                       kMaskWindow  lo = max(0, i - size + 1)
 //                       kMaskChunk   lo = floor(i / size) * size   (chunks counted from the sequence's start)
 //                     score = (q . k) * scale * temp[h];  p_j = exp(score_j) / (sum_j' exp(score_j') + exp(sink[h]))
-//                     (the sink adds to the denominator only: no key, no value, not scaled). Positions do
-//                     not enter the scores.
+//                     (the sink adds to the denominator only: no key, no value, not scaled). Positions enter
+//                     the scores only through an optional distance penalty: with r1 / r2 the score of key j
+//                     loses r1[h] * ln(1 + r2[h] * (i - j)). With `gate` head h's output is multiplied by
+//                     sigmoid(gate[t][h]). `vmode` chooses the values a query head weighs: kValuesOwn its own
+//                     key/value head's (output [T][H][dv]), kValuesAll the values of all G heads side by side
+//                     (output [T][H][G dv]: what mixing the heads' weight maps after the softmax needs),
+//                     c >= 0 head c's for every query head.
+//   talk_mix          out[t][h] = sigmoid(gate[t][h]) * sum_g talk[h][g] * o_all[t][g][c(h)], c(h) = h / (H / G)
+//   head_norm_rope_cache  per-head RMS norm of q and k (one weight of a head's size for all heads), pairwise
+//                     rotation of each head's first entries by a (cos, sin) table row of the token's position,
+//                     q to a dense tensor, k / v to the cache rows slot_mapping[t]
 //
 // Activations / caches are T = float or bf16; norms, scores, probabilities and the accumulators are fp32.
 #include "mixers_common.h"
@@ -18,6 +27,7 @@
 namespace xgm {
 
 constexpr int kMaskCausal = 0, kMaskWindow = 1, kMaskChunk = 2;
+constexpr int kValuesOwn = -1, kValuesAll = -2;
 
 __device__ __forceinline__ int first_visible(int mask, int size, int pos) {
   if (mask == kMaskWindow) return max(0, pos - size + 1);
@@ -71,8 +81,12 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     const T* __restrict__ q, const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int32_t* __restrict__ block_tables, int bt_width, int bs, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ token_seq, const float* __restrict__ temp, const float* __restrict__ sink,
-    T* __restrict__ out, int H, int G, int dk, int dv, int mask, int size, float scale, int KT) {
+    T* __restrict__ out, int H, int G, int dk, int dv_head, int mask, int size, float scale, int KT,
+    const T* __restrict__ gate, int64_t ld_gate, const float* __restrict__ r1, const float* __restrict__ r2, int vmode) {
   extern __shared__ float smem[];
+  // dv: value columns per query head; voff: where they start in a cached row of G * dv_head values
+  const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
+  const int voff = vmode == kValuesAll ? 0 : (vmode >= 0 ? vmode : (int)blockIdx.y) * dv_head;
   const int ldk = dk + 1, ldv = dv + 1;
   float* ktile = smem;                           // [KT][dk + 1]
   float* vtile = ktile + (size_t)KT * ldk;       // [KT][dv + 1]
@@ -92,11 +106,13 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
   }
   const int pos = positions[t];
   const int j0 = first_visible(mask, size, pos);
-  float m[kQPW], l[kQPW], acc[kQPW][NR];
+  float m[kQPW], l[kQPW], acc[kQPW][NR], pen1[kQPW], pen2[kQPW];
 #pragma unroll
   for (int a = 0; a < kQPW; ++a) {
     const int r = r0 + wave + 4 * a;
     const int h = g * rep + min(r, rep - 1);
+    pen1[a] = r1 ? r1[h] : 0.f;
+    pen2[a] = r1 ? r2[h] : 0.f;
     float* qh = qs + (wave + 4 * a) * dk;
     const float sc = scale * (temp ? temp[h] : 1.f);
     for (int d = lane; d < dk; d += 64) qh[d] = r < rep ? ldf(q + ((int64_t)t * H + h) * dk + d) * sc : 0.f;
@@ -116,7 +132,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
       const int key = k0 + jj;
       const int64_t row = (int64_t)bt[key / bs] * bs + key % bs;
       const T* ks = kcache + (row * G + g) * dk;
-      const T* vs = vcache + (row * G + g) * dv;
+      const T* vs = vcache + row * G * dv_head + voff;
       for (int d = lane; d < dk; d += 64) ktile[jj * ldk + d] = ldf(ks + d);
       for (int d = lane; d < dv; d += 64) vtile[jj * ldv + d] = ldf(vs + d);
     }
@@ -131,6 +147,7 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
         for (int d = part; d < dk; d += LPK) sc += qh[d] * kr[d];
       }
       for (int o = 1; o < LPK; o <<= 1) sc += __shfl_xor(sc, o, 64);
+      if (r1 && kj < n) sc -= pen1[a] * log1pf(pen2[a] * (float)(pos - (k0 + kj)));
       if (kj >= n) sc = -INFINITY;
       const float mn = fmaxf(m[a], wave_max(sc));
       const float p = kj < n ? expf(sc - mn) : 0.f;
@@ -153,7 +170,8 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
   for (int a = 0; a < kQPW; ++a) {
     const int r = r0 + wave + 4 * a;
     if (r >= rep) continue;
-    const float inv = 1.f / l[a];
+    float inv = 1.f / l[a];
+    if (gate) inv *= sigmoidf(ldf(gate + (int64_t)t * ld_gate + g * rep + r));
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       const int d = lane + 64 * i;
@@ -177,9 +195,12 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int32_t* __restrict__ block_tables, int bt_width, int bs, const int32_t* __restrict__ qsl,
     const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, const float* __restrict__ temp,
-    const float* __restrict__ sink, bf16* __restrict__ out, int H, int G, int dk, int dv, int mask, int size, float scale,
-    int RH, int head_slots, float* __restrict__ part_o, float* __restrict__ part_ml, int Ttot) {
+    const float* __restrict__ sink, bf16* __restrict__ out, int H, int G, int dk, int dv_head, int mask, int size,
+    float scale, int RH, int head_slots, float* __restrict__ part_o, float* __restrict__ part_ml, int Ttot,
+    const bf16* __restrict__ gate, int64_t ld_gate, const float* __restrict__ r1, const float* __restrict__ r2, int vmode) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  // dv: value columns per query head; voff: where they start in a cached row of G * dv_head values
+  const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
   const int LDK = dk + 8, LDV = dv + 8;
   uint16_t* ktile = lds;                 // [kKT][LDK]
   uint16_t* vtile = lds + kKT * LDK;     // [kKT][LDV]
@@ -205,6 +226,8 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
   const bool wave_on = head_slots ? wave * 16 < rep : (hr < rep && t0 + (wave / RH) * 16 < qn);
   const bool valid = wave_on && hr < rep && tok < qn;
   const int head = g * rep + min(hr, rep - 1);
+  const int voff = vmode == kValuesAll ? 0 : (vmode >= 0 ? vmode : g) * dv_head;
+  const float pen1 = r1 ? r1[head] : 0.f, pen2 = r1 ? r2[head] : 0.f;
   const int ctx = seq_lens[s] - qn;
   const int pos_q = ctx + min(tok, qn - 1);
   const int lo_q = first_visible(mask, size, pos_q);
@@ -246,7 +269,7 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
     const bool ok = kabs <= pos_last;
     const int64_t row = ok ? (int64_t)bt[kabs / bs] * bs + kabs % bs : 0;
     const bf16* ks = kcache + (row * G + g) * dk;
-    const bf16* vs = vcache + (row * G + g) * dv;
+    const bf16* vs = vcache + row * G * dv_head + voff;
 #pragma unroll
     for (int it = 0; it < NKK_MAX; ++it) {
       const int ch = squad + 4 * it;
@@ -294,6 +317,7 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
       for (int r = 0; r < 4; ++r) {
         const int kabs = k0 + n * 16 + kg * 4 + r;
         float v = sacc[n][r] * sc_h;
+        if (r1) v -= pen1 * __logf(1.f + pen2 * (float)max(pos_q - kabs, 0));
         if (!valid || kabs > pos_q || kabs < lo_q) v = -INFINITY;
         sacc[n][r] = v;
         mx = fmaxf(mx, v);
@@ -351,7 +375,8 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
       if (mt < nmt)
         *reinterpret_cast<float4*>(part_o + row * dv + mt * 16 + 4 * kg) = make_float4(o[mt][0], o[mt][1], o[mt][2], o[mt][3]);
   } else if (valid) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float inv = l > 0.f ? 1.f / l : 0.f;
+    if (gate) inv *= sigmoidf(bf2f(gate[(int64_t)(q0 + tok) * ld_gate + head]));
     bf16* op = out + ((int64_t)(q0 + tok) * H + head) * dv;
 #pragma unroll
     for (int mt = 0; mt < NMT_MAX; ++mt)
@@ -367,7 +392,7 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
 // merge the key shares of a single-token step: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s
 __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                 const int32_t* __restrict__ slots, bf16* __restrict__ out, int Ttot, int H,
-                                                int dv, int nsplit) {
+                                                int dv, int nsplit, const bf16* __restrict__ gate, int64_t ld_gate) {
   const int t = blockIdx.x, h = blockIdx.y;
   if (slots[t] < 0) return;  // single-token steps: row t is sequence t (its output row was zeroed)
   float M = -INFINITY;
@@ -378,7 +403,8 @@ __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o
     const float ms = part_ml[2 * row];
     if (ms != -INFINITY) L += __expf(ms - M) * part_ml[2 * row + 1];
   }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
+  float inv = L > 0.f ? 1.f / L : 0.f;
+  if (gate) inv *= sigmoidf(bf2f(gate[(int64_t)t * ld_gate + h]));
   for (int d = threadIdx.x; d < dv; d += blockDim.x) {
     float acc = 0.f;
     for (int sp = 0; sp < nsplit; ++sp) {
@@ -388,6 +414,71 @@ __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o
     }
     out[((int64_t)t * H + h) * dv + d] = f2bf(acc * inv);
   }
+}
+
+// ------------------------------------------------------------------ heads' weight maps mixed after the softmax
+// o_all[t][g][c][:] = p_g V_c for every query head g and key/value head c; head h's mixed weights
+// sum_g talk[h][g] p_g applied to the values of its own key/value head c(h) are sum_g talk[h][g] o_all[t][g][c(h)].
+template <typename T>
+__global__ __launch_bounds__(256) void talk_mix_kernel(const T* __restrict__ o_all, const float* __restrict__ talk,
+                                                       const T* __restrict__ gate, int64_t ld_gate, T* __restrict__ out,
+                                                       int H, int G, int dv) {
+  const int t = blockIdx.x;
+  const int rep = H / G;
+  const T* row = o_all + (int64_t)t * H * G * dv;
+  for (int e = threadIdx.x; e < H * dv; e += blockDim.x) {
+    const int h = e / dv, d = e % dv;
+    const int c = h / rep;
+    float acc = 0.f;
+    for (int g = 0; g < H; ++g) acc += talk[h * H + g] * ldf(row + ((int64_t)g * G + c) * dv + d);
+    if (gate) acc *= sigmoidf(ldf(gate + (int64_t)t * ld_gate + h));
+    stf(out + (int64_t)t * H * dv + e, acc);
+  }
+}
+
+// ------------------------------------------------------------------ per-head norm + rotation -> q, cache rows
+// One workgroup per token; a wave takes the heads (H query heads, then G key heads) round robin. A lane owns the
+// entries d = lane, lane + 64, ... of a head; the partner of a rotated entry is re-read (it is in the same row).
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(
+    const TI* __restrict__ src, int64_t ld, int H, int G, int dk, int dv, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, const float* __restrict__ rot, int rot_rows, int rot_dims,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_mapping, TO* __restrict__ q_out,
+    TO* __restrict__ kcache, TO* __restrict__ vcache) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const TI* row = src + (int64_t)t * ld;
+  const int slot = slot_mapping[t];
+  const int nq = H * dk, nk = G * dk, nv = G * dv;
+  const float* cs = nullptr;
+  if (rot && rot_dims > 0) cs = rot + (int64_t)min(max(positions[t], 0), rot_rows - 1) * rot_dims;  // [rot_dims / 2][2]
+  for (int hd = wave; hd < H + G; hd += nw) {
+    const bool is_q = hd < H;
+    if (!is_q && slot < 0) continue;   // padding row: nothing is cached
+    const TI* v = row + (is_q ? hd * dk : nq + (hd - H) * dk);
+    const float* w = is_q ? wq : wk;
+    TO* dst = is_q ? q_out + (int64_t)t * nq + hd * dk : kcache + (int64_t)slot * nk + (hd - H) * dk;
+    float r = 1.f;
+    if (w) {
+      float ss = 0.f;
+      for (int d = lane; d < dk; d += 64) {
+        const float a = ldf(v + d);
+        ss += a * a;
+      }
+      r = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
+    }
+    for (int d = lane; d < dk; d += 64) {
+      float a = ldf(v + d) * r * (w ? w[d] : 1.f);
+      if (cs && d < rot_dims) {
+        const float b = ldf(v + (d ^ 1)) * r * (w ? w[d ^ 1] : 1.f);
+        const float c = cs[d & ~1], sn = cs[(d & ~1) + 1];
+        a = (d & 1) ? a * c + b * sn : a * c - b * sn;   // (u, v) -> (u c - v s, v c + u s)
+      }
+      stf(dst + d, a);
+    }
+  }
+  if (slot >= 0)
+    for (int c = threadIdx.x; c < nv; c += blockDim.x) stf(vcache + (int64_t)slot * nv + c, ldf(row + nq + nk + c));
 }
 
 // ================================================================== host launchers
@@ -402,8 +493,10 @@ void qk_norm_cache(const void* proj, bool f32, int64_t ld, int nq, int nk, int n
 template <typename T, int NR>
 static int launch_masked_attention(const void* q, const void* kcache, const void* vcache, const int32_t* block_tables,
                                    int bt_width, int bs, const int32_t* positions, const int32_t* token_seq,
-                                   const float* temp, const float* sink, void* out, int T_, int H, int G, int dk, int dv,
-                                   int mask, int size, float scale, hipStream_t st) {
+                                   const float* temp, const float* sink, void* out, int T_, int H, int G, int dk,
+                                   int dv_head, int mask, int size, float scale, const void* gate, int64_t ld_gate,
+                                   const float* r1, const float* r2, int vmode, hipStream_t st) {
+  const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
   int KT = 64;
   auto bytes = [&](int kt) { return ((size_t)kt * (dk + dv + 2) + (size_t)4 * kQPW * dk) * sizeof(float); };
   while (KT > 4 && bytes(KT) > 60 * 1024) KT >>= 1;
@@ -412,21 +505,25 @@ static int launch_masked_attention(const void* q, const void* kcache, const void
   dim3 grid(T_, G, (rep + 4 * kQPW - 1) / (4 * kQPW));
   masked_attention_kernel<T, NR><<<grid, 256, bytes(KT), st>>>((const T*)q, (const T*)kcache, (const T*)vcache,
                                                                block_tables, bt_width, bs, positions, token_seq, temp,
-                                                               sink, (T*)out, H, G, dk, dv, mask, size, scale, KT);
+                                                               sink, (T*)out, H, G, dk, dv_head, mask, size, scale, KT,
+                                                               (const T*)gate, ld_gate, r1, r2, vmode);
   return 0;
 }
 
 int masked_attention(const void* q, bool f32, const void* kcache, const void* vcache, const int32_t* block_tables,
                      int bt_width, int bs, const int32_t* positions, const int32_t* token_seq, const float* temp,
-                     const float* sink, void* out, int T_, int H, int G, int dk, int dv, int mask, int size, float scale,
+                     const float* sink, void* out, int T_, int H, int G, int dk, int dv_head, int mask, int size,
+                     float scale, const void* gate, int64_t ld_gate, const float* r1, const float* r2, int vmode,
                      hipStream_t st) {
   if (T_ <= 0) return 0;
-  if (G <= 0 || H % G != 0 || dk <= 0 || dv <= 0 || dv > 512 || mask < 0 || mask > 2 || (mask != kMaskCausal && size < 1))
+  const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
+  if (G <= 0 || H % G != 0 || dk <= 0 || dv <= 0 || dv > 512 || mask < 0 || mask > 2 ||
+      (mask != kMaskCausal && size < 1) || vmode < kValuesAll || vmode >= G || (r1 && !r2))
     return -1;
 #define XGM_MA(NR)                                                                                                     \
   XGM_DISPATCH_T(f32, return (launch_masked_attention<T, NR>(q, kcache, vcache, block_tables, bt_width, bs, positions, \
-                                                             token_seq, temp, sink, out, T_, H, G, dk, dv, mask, size, \
-                                                             scale, st));)
+                                                             token_seq, temp, sink, out, T_, H, G, dk, dv_head, mask,  \
+                                                             size, scale, gate, ld_gate, r1, r2, vmode, st));)
   if (dv <= 64) { XGM_MA(1) }
   if (dv <= 128) { XGM_MA(2) }
   if (dv <= 256) { XGM_MA(4) }
@@ -437,11 +534,13 @@ int masked_attention(const void* q, bool f32, const void* kcache, const void* vc
 
 int masked_attention_mfma(const void* q, const void* kcache, const void* vcache, const int32_t* block_tables, int bt_width,
                           int bs, const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, const float* temp,
-                          const float* sink, void* out, int T_, int ns, int max_q, int H, int G, int dk, int dv, int mask,
-                          int size, float scale, int nsplit, float* part_o, float* part_ml, hipStream_t st) {
+                          const float* sink, void* out, int T_, int ns, int max_q, int H, int G, int dk, int dv_head,
+                          int mask, int size, float scale, int nsplit, float* part_o, float* part_ml, const void* gate,
+                          int64_t ld_gate, const float* r1, const float* r2, int vmode, hipStream_t st) {
   if (T_ <= 0 || ns <= 0 || max_q <= 0) return 0;
-  if (G <= 0 || H % G != 0 || dk % 32 != 0 || dv % 16 != 0 || dk > 128 || dv > 128 || mask < 0 || mask > 2 ||
-      (mask != kMaskCausal && size < 1))
+  const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
+  if (G <= 0 || H % G != 0 || dk % 32 != 0 || dv % 16 != 0 || dk > 128 || dv > 256 || mask < 0 || mask > 2 ||
+      (mask != kMaskCausal && size < 1) || vmode < kValuesAll || vmode >= G || (r1 && !r2))
     return -1;
   const int rep = H / G;
   const int RH = rep >= 4 ? 4 : rep >= 2 ? 2 : 1;
@@ -456,16 +555,43 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
 #define XGM_MM(NKK, NMT)                                                                                              \
   masked_attention_mfma_kernel<NKK, NMT><<<grid, 256, lds, st>>>((const bf16*)q, (const bf16*)kcache,                 \
                                                                  (const bf16*)vcache, block_tables, bt_width, bs, qsl, \
-                                                                 seq_lens, slots, temp, sink, (bf16*)out, H, G, dk, dv, \
-                                                                 mask, size, scale, RH, head_slots, part_o, part_ml,   \
-                                                                 T_);                                                  \
+                                                                 seq_lens, slots, temp, sink, (bf16*)out, H, G, dk,    \
+                                                                 dv_head, mask, size, scale, RH, head_slots, part_o,   \
+                                                                 part_ml, T_, (const bf16*)gate, ld_gate, r1, r2,      \
+                                                                 vmode);                                               \
   if (nsplit > 1)                                                                                                     \
-    masked_attention_combine_kernel<<<dim3(T_, H), 64, 0, st>>>(part_o, part_ml, slots, (bf16*)out, T_, H, dv, nsplit); \
+    masked_attention_combine_kernel<<<dim3(T_, H), 64, 0, st>>>(part_o, part_ml, slots, (bf16*)out, T_, H, dv, nsplit, \
+                                                                (const bf16*)gate, ld_gate);                          \
   return 0;
   if (dk <= 64 && dv <= 64) { XGM_MM(2, 4) }
   if (dk <= 128 && dv <= 128) { XGM_MM(4, 8) }
+  if (dk <= 128 && dv <= 256) { XGM_MM(4, 16) }
   return -2;
 #undef XGM_MM
+}
+
+void talk_mix(const void* o_all, bool f32, const float* talk, const void* gate, int64_t ld_gate, void* out, int T_, int H,
+              int G, int dv, hipStream_t st) {
+  if (T_ <= 0) return;
+  XGM_DISPATCH_T(f32, talk_mix_kernel<T><<<T_, 256, 0, st>>>((const T*)o_all, talk, (const T*)gate, ld_gate, (T*)out, H, G,
+                                                              dv);)
+}
+
+void head_norm_rope_cache(const void* src, bool src_f32, int64_t ld, int H, int G, int dk, int dv, const float* wq,
+                          const float* wk, float eps, const float* rot, int rot_rows, int rot_dims,
+                          const int32_t* positions, const int32_t* slot_mapping, void* q_out, void* kcache, void* vcache,
+                          bool out_f32, int T_, hipStream_t st) {
+  if (T_ <= 0) return;
+#define XGM_HN(TI, TO)                                                                                               \
+  head_norm_rope_cache_kernel<TI, TO><<<T_, 256, 0, st>>>((const TI*)src, ld, H, G, dk, dv, wq, wk, eps, rot, rot_rows, \
+                                                          rot_dims, positions, slot_mapping, (TO*)q_out, (TO*)kcache,  \
+                                                          (TO*)vcache);
+  if (src_f32) {
+    if (out_f32) { XGM_HN(float, float) } else { XGM_HN(float, bf16) }
+  } else {
+    if (out_f32) { XGM_HN(bf16, float) } else { XGM_HN(bf16, bf16) }
+  }
+#undef XGM_HN
 }
 
 }  // namespace xgm

@@ -1,0 +1,164 @@
+// Gated linear recurrence with one decay per state row (gated linear attention; with k = 1 - f the
+// forget gate also decides what is written), carried per sequence slot.
+//
+//   lower_bound_gates  from a fused projection row: q = silu(z_q);  f = l + (1 - l) * sigmoid(z_f + b)
+//                      (a forget gate bounded below by l, per channel), both fp32
+//   gated_linear_scan  per head, state S [dk x dv] fp32 per (slot, head):
+//                        S_t = diag(f_t) S_(t-1) + k_t v_t^T        (k_t = 1 - f_t when k == nullptr)
+//                        o_t = S_t^T q_t
+//
+// One workgroup = (sequence, head, 64 state columns), NW waves: lane p owns column p, wave w owns rows
+// [w * NI, (w + 1) * NI) of it in registers. f / k / q / v of TT tokens at a time are staged in LDS (two buffers:
+// the next tile's global loads are issued before the current tile's steps and stored after them). Per token
+// a wave does 2 FMAs per owned state element; the waves' partial sums of o meet in LDS once per tile, in
+// wave order.
+#include "mixers_common.h"
+
+namespace xgm {
+
+template <typename T>
+__global__ void lower_bound_gates_kernel(const T* __restrict__ proj, int64_t ld, int off_q, int off_f, int n,
+                                         const float* __restrict__ f_bias, const float* __restrict__ lower,
+                                         float* __restrict__ q, float* __restrict__ f, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / n;
+  const int c = (int)(i % n);
+  const T* row = proj + t * ld;
+  q[i] = siluf(ldf(row + off_q + c));
+  const float l = lower[c];
+  f[i] = l + (1.f - l) * sigmoidf(ldf(row + off_f + c) + (f_bias ? f_bias[c] : 0.f));
+}
+
+constexpr int kGlaCols = 64;   // state columns per workgroup
+
+template <typename T, int NI, int TT, int NW>
+__global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
+    const float* __restrict__ q, const float* __restrict__ f, const float* __restrict__ k, const T* __restrict__ v,
+    int64_t ld_v, float* __restrict__ state, const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens,
+    const int32_t* __restrict__ slots, float* __restrict__ o, int H, int dk, int dv) {
+  constexpr int NB = NW * NI;                // padded state rows
+  constexpr int NTH = 64 * NW;
+  constexpr int ROW = 3 * NB + kGlaCols;     // staged floats per token: [f | k | q | v]
+  constexpr int PER = (TT * ROW + NTH - 1) / NTH;
+  __shared__ __attribute__((aligned(16))) float stage[2][TT][ROW];
+  __shared__ float opart[TT][NW][kGlaCols];
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int q0 = qsl[s], qn = qsl[s + 1] - q0, slot = slots[s];
+  if (slot < 0 || qn <= 0) return;
+  const int ctx = seq_lens[s] - qn;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int p0 = blockIdx.z * kGlaCols, p = p0 + lane;
+  const bool pok = p < dv;
+  const int nqk = H * dk, nv = H * dv;
+  float* Sg = state + (((int64_t)slot * H + h) * dk) * dv;
+  float S[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int n = wave * NI + i;
+    S[i] = (ctx > 0 && pok && n < dk) ? Sg[(int64_t)n * dv + p] : 0.f;
+  }
+  float pre[PER];
+  auto fetch = [&](int t0) {  // global loads of the tile starting at token t0 (zeros past the end / the sizes)
+    const int nt = min(TT, qn - t0);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = threadIdx.x + NTH * j;
+      const int tt = e / ROW, c = e % ROW;
+      float val = 0.f;
+      if (tt < nt) {
+        const int64_t tok = q0 + t0 + tt;
+        if (c < NB) {
+          if (c < dk) val = f[tok * nqk + h * dk + c];
+        } else if (c < 2 * NB) {
+          const int cc = c - NB;
+          if (cc < dk) val = k ? k[tok * nqk + h * dk + cc] : 1.f - f[tok * nqk + h * dk + cc];
+        } else if (c < 3 * NB) {
+          const int cc = c - 2 * NB;
+          if (cc < dk) val = q[tok * nqk + h * dk + cc];
+        } else if (p0 + c - 3 * NB < dv) {
+          val = ldf(v + tok * ld_v + h * dv + p0 + c - 3 * NB);
+        }
+      }
+      pre[j] = val;
+    }
+  };
+  auto commit = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = threadIdx.x + NTH * j;
+      if (e < TT * ROW) (&stage[buf][0][0])[e] = pre[j];
+    }
+  };
+  fetch(0);
+  commit(0);
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = 0; t0 < qn; t0 += TT, buf ^= 1) {
+    const int nt = min(TT, qn - t0);
+    const bool more = t0 + TT < qn;
+    if (more) fetch(t0 + TT);
+    for (int tt = 0; tt < nt; ++tt) {
+      const float* fr = &stage[buf][tt][wave * NI];
+      const float* kr = &stage[buf][tt][NB + wave * NI];
+      const float* qr = &stage[buf][tt][2 * NB + wave * NI];
+      const float vv = stage[buf][tt][3 * NB + lane];
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        S[i] = fr[i] * S[i] + kr[i] * vv;
+        acc += S[i] * qr[i];
+      }
+      opart[tt][wave][lane] = acc;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * kGlaCols; e += NTH) {
+      const int tt = e / kGlaCols, c = e % kGlaCols;
+      if (p0 + c < dv) {
+        float val = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) val += opart[tt][w][c];
+        o[(int64_t)(q0 + t0 + tt) * nv + h * dv + p0 + c] = val;
+      }
+    }
+    if (more) commit(buf ^ 1);
+    __syncthreads();
+  }
+  if (pok) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = wave * NI + i;
+      if (n < dk) Sg[(int64_t)n * dv + p] = S[i];
+    }
+  }
+}
+
+// ================================================================== host launchers
+void lower_bound_gates(const void* proj, bool f32, int64_t ld, int off_q, int off_f, int n, const float* f_bias,
+                       const float* lower, float* q, float* f, int T_, hipStream_t st) {
+  if (T_ <= 0 || n <= 0) return;
+  const int64_t total = (int64_t)T_ * n;
+  XGM_DISPATCH_T(f32, lower_bound_gates_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(
+                          (const T*)proj, ld, off_q, off_f, n, f_bias, lower, q, f, total);)
+}
+
+int gated_linear_scan(const float* q, const float* f, const float* k, const void* v, bool v_f32, int64_t ld_v, float* state,
+                      const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, float* o, int ns, int H, int dk,
+                      int dv, hipStream_t st) {
+  if (ns <= 0) return 0;
+  if (H <= 0 || dk < 1 || dk > 256 || dv < 1) return -1;
+  dim3 grid(ns, H, (dv + kGlaCols - 1) / kGlaCols);
+#define XGM_GL(NI, TT, NW)                                                                                              \
+  XGM_DISPATCH_T(v_f32, gated_linear_scan_kernel<T, NI, TT, NW><<<grid, 64 * NW, 0, st>>>(q, f, k, (const T*)v, ld_v, state, \
+                                                                                          qsl, seq_lens, slots, o, H, dk, \
+                                                                                          dv);)                         \
+  return 0;
+  if (dk <= 16) { XGM_GL(4, 16, 4) }
+  if (dk <= 32) { XGM_GL(8, 16, 4) }
+  if (dk <= 64) { XGM_GL(8, 8, 8) }
+  if (dk <= 128) { XGM_GL(16, 8, 8) }
+  XGM_GL(32, 4, 8)
+#undef XGM_GL
+}
+
+}  // namespace xgm

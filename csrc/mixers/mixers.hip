@@ -24,18 +24,19 @@
 namespace xgm {
 
 // ------------------------------------------------------------------ embedding
-// pos_table != nullptr: + pos_table[positions[t]] (a learned vector per position, rows outside the table add nothing)
+// out = table[id] * scale; pos_table != nullptr: + pos_table[positions[t]] (a learned vector per position, unscaled;
+// rows outside the table add nothing)
 template <typename TW>
 __global__ void embed_rows_kernel(const int32_t* __restrict__ ids, const TW* __restrict__ table, float* __restrict__ out,
                                   int W, int V, const TW* __restrict__ pos_table, const int32_t* __restrict__ positions,
-                                  int P) {
+                                  int P, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   const bool ok = id >= 0 && id < V;
   const int p = pos_table ? positions[t] : -1;
   const bool pk = p >= 0 && p < P;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float v = ok ? ldf(table + (int64_t)id * W + c) : 0.f;
+    float v = ok ? ldf(table + (int64_t)id * W + c) * scale : 0.f;
     if (pk) v += ldf(pos_table + (int64_t)p * W + c);
     out[(int64_t)t * W + c] = v;
   }
@@ -848,10 +849,10 @@ __global__ void heads_to_rows_kernel(const T* __restrict__ in, T* __restrict__ o
 
 // ================================================================== host launchers
 void embed_rows(const int32_t* ids, const void* table, bool f32, float* out, int T_, int W, int V, const void* pos_table,
-                const int32_t* positions, int P, hipStream_t st) {
+                const int32_t* positions, int P, float scale, hipStream_t st) {
   if (T_ <= 0) return;
   XGM_DISPATCH_T(f32, embed_rows_kernel<T><<<T_, 256, 0, st>>>(ids, (const T*)table, out, W, V, (const T*)pos_table,
-                                                                positions, P);)
+                                                                positions, P, scale);)
 }
 
 void causal_conv(const void* x, bool in_f32, int64_t ld_in, const float* w, const float* bias, float* state,

@@ -10,7 +10,8 @@
 namespace py = pybind11;
 
 namespace xgm {
-void embed_rows(const int32_t*, const void*, bool, float*, int, int, int, const void*, const int32_t*, int, hipStream_t);
+void embed_rows(const int32_t*, const void*, bool, float*, int, int, int, const void*, const int32_t*, int, float,
+                hipStream_t);
 void causal_conv(const void*, bool, int64_t, const float*, const float*, float*, const int32_t*, const int32_t*,
                  const int32_t*, void*, bool, int, int, int, int, bool, bool, hipStream_t);
 void residual_norm(float*, const void*, int64_t, const float*, const void*, int64_t, const float*, const float*, bool,
@@ -19,13 +20,24 @@ void qk_norm_cache(const void*, bool, int64_t, int, int, int, const float*, cons
                    void*, void*, int, hipStream_t);
 int masked_attention(const void*, bool, const void*, const void*, const int32_t*, int, int, const int32_t*,
                      const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
-                     hipStream_t);
+                     const void*, int64_t, const float*, const float*, int, hipStream_t);
 int masked_attention_mfma(const void*, const void*, const void*, const int32_t*, int, int, const int32_t*, const int32_t*,
                           const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, int, int,
-                          float, int, float*, float*, hipStream_t);
+                          float, int, float*, float*, const void*, int64_t, const float*, const float*, int, hipStream_t);
+void talk_mix(const void*, bool, const float*, const void*, int64_t, void*, int, int, int, int, hipStream_t);
+void head_norm_rope_cache(const void*, bool, int64_t, int, int, int, int, const float*, const float*, float, const float*,
+                          int, int, const int32_t*, const int32_t*, void*, void*, void*, bool, int, hipStream_t);
+int post_norm_residual(float*, const void*, bool, int64_t, const float*, const void*, int64_t, const float*, const float*,
+                       const float*, float, const float*, const float*, float, float, void*, bool, int, int, hipStream_t);
+void relu2(const void*, bool, const float*, void*, int64_t, int, hipStream_t);
+void lower_bound_gates(const void*, bool, int64_t, int, int, int, const float*, const float*, float*, float*, int,
+                       hipStream_t);
+int gated_linear_scan(const float*, const float*, const float*, const void*, bool, int64_t, float*, const int32_t*,
+                      const int32_t*, const int32_t*, float*, int, int, int, int, hipStream_t);
 int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, const float*, const float*, float*,
              const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, int, int, hipStream_t);
-void gated_group_norm(const float*, const void*, bool, int64_t, const float*, float, void*, int, int, int, hipStream_t);
+void gated_group_norm(const float*, const void*, bool, int64_t, const float*, int, float, void*, int, int, int,
+                      hipStream_t);
 void glu_act(const void*, bool, int64_t, void*, int, int, int, float, float, hipStream_t);
 int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, hipStream_t);
 int moe_align(const int32_t*, int, int, int, int, int32_t*, int32_t*, int32_t*, hipStream_t);
@@ -63,10 +75,10 @@ static void check(int rc, const char* what) {
 
 PYBIND11_MODULE(_mixers, m) {
   m.def("embed_rows", [](uintptr_t ids, uintptr_t table, bool f32, uintptr_t out, int T, int W, int V, uintptr_t pos_table,
-                         uintptr_t positions, int Pn, uintptr_t st) {
+                         uintptr_t positions, int Pn, float scale, uintptr_t st) {
     if (pos_table && !positions) throw std::invalid_argument("embed_rows: a position table needs positions");
     xgm::embed_rows(P<const int32_t>(ids), P<const void>(table), f32, P<float>(out), T, W, V, P<const void>(pos_table),
-                    P<const int32_t>(positions), Pn, S(st));
+                    P<const int32_t>(positions), Pn, scale, S(st));
     check(0, "embed_rows");
   });
   m.def("causal_conv", [](uintptr_t x, bool in_f32, int64_t ld_in, uintptr_t w, uintptr_t bias, uintptr_t state,
@@ -98,24 +110,84 @@ PYBIND11_MODULE(_mixers, m) {
   });
   m.def("masked_attention", [](uintptr_t q, bool f32, uintptr_t kc, uintptr_t vc, uintptr_t bt, int bt_width, int bs,
                                uintptr_t pos, uintptr_t token_seq, uintptr_t temp, uintptr_t sink, uintptr_t out, int T,
-                               int H, int G, int dk, int dv, int mask, int size, float scale, uintptr_t st) {
-    if (bs < 1 || bt_width < 1) throw std::invalid_argument("masked_attention: inconsistent sizes");
+                               int H, int G, int dk, int dv, int mask, int size, float scale, uintptr_t gate,
+                               int64_t ld_gate, uintptr_t r1, uintptr_t r2, int vmode, uintptr_t st) {
+    if (bs < 1 || bt_width < 1 || (gate && ld_gate < H))
+      throw std::invalid_argument("masked_attention: inconsistent sizes");
     int rc = xgm::masked_attention(P<const void>(q), f32, P<const void>(kc), P<const void>(vc), P<const int32_t>(bt),
                                    bt_width, bs, P<const int32_t>(pos), P<const int32_t>(token_seq), P<const float>(temp),
-                                   P<const float>(sink), P<void>(out), T, H, G, dk, dv, mask, size, scale, S(st));
+                                   P<const float>(sink), P<void>(out), T, H, G, dk, dv, mask, size, scale,
+                                   P<const void>(gate), ld_gate, P<const float>(r1), P<const float>(r2), vmode, S(st));
     check(rc, "masked_attention");
   });
   m.def("masked_attention_mfma", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int bt_width, int bs,
                                     uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t temp, uintptr_t sink,
                                     uintptr_t out, int T, int ns, int max_q, int H, int G, int dk, int dv, int mask,
                                     int size, float scale, int nsplit, uintptr_t part_o, uintptr_t part_ml,
+                                    uintptr_t gate, int64_t ld_gate, uintptr_t r1, uintptr_t r2, int vmode,
                                     uintptr_t st) {
-    if (bs < 1 || bt_width < 1 || nsplit < 1) throw std::invalid_argument("masked_attention_mfma: inconsistent sizes");
+    if (bs < 1 || bt_width < 1 || nsplit < 1 || (gate && ld_gate < H))
+      throw std::invalid_argument("masked_attention_mfma: inconsistent sizes");
     int rc = xgm::masked_attention_mfma(P<const void>(q), P<const void>(kc), P<const void>(vc), P<const int32_t>(bt),
                                         bt_width, bs, P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
                                         P<const float>(temp), P<const float>(sink), P<void>(out), T, ns, max_q, H, G, dk,
-                                        dv, mask, size, scale, nsplit, P<float>(part_o), P<float>(part_ml), S(st));
+                                        dv, mask, size, scale, nsplit, P<float>(part_o), P<float>(part_ml),
+                                        P<const void>(gate), ld_gate, P<const float>(r1), P<const float>(r2), vmode,
+                                        S(st));
     check(rc, "masked_attention_mfma");
+  });
+  m.def("talk_mix", [](uintptr_t o_all, bool f32, uintptr_t talk, uintptr_t gate, int64_t ld_gate, uintptr_t out, int T,
+                       int H, int G, int dv, uintptr_t st) {
+    if (H < 1 || G < 1 || H % G || dv < 1 || (gate && ld_gate < H))
+      throw std::invalid_argument("talk_mix: inconsistent sizes");
+    xgm::talk_mix(P<const void>(o_all), f32, P<const float>(talk), P<const void>(gate), ld_gate, P<void>(out), T, H, G, dv,
+                  S(st));
+    check(0, "talk_mix");
+  });
+  m.def("head_norm_rope_cache", [](uintptr_t src, bool src_f32, int64_t ld, int H, int G, int dk, int dv, uintptr_t wq,
+                                   uintptr_t wk, float eps, uintptr_t rot, int rot_rows, int rot_dims, uintptr_t pos,
+                                   uintptr_t slot_mapping, uintptr_t q_out, uintptr_t kc, uintptr_t vc, bool out_f32, int T,
+                                   uintptr_t st) {
+    if (H < 1 || G < 1 || dk < 1 || dv < 1 || ld < (int64_t)(H + G) * dk + (int64_t)G * dv || rot_dims < 0 ||
+        rot_dims > dk || (rot_dims & 1) || (rot && rot_dims > 0 && rot_rows < 1))
+      throw std::invalid_argument("head_norm_rope_cache: inconsistent sizes");
+    xgm::head_norm_rope_cache(P<const void>(src), src_f32, ld, H, G, dk, dv, P<const float>(wq), P<const float>(wk), eps,
+                              P<const float>(rot), rot_rows, rot_dims, P<const int32_t>(pos),
+                              P<const int32_t>(slot_mapping), P<void>(q_out), P<void>(kc), P<void>(vc), out_f32, T, S(st));
+    check(0, "head_norm_rope_cache");
+  });
+  m.def("post_norm_residual", [](uintptr_t x, uintptr_t y, bool y_f32, int64_t ldy, uintptr_t y_bias, uintptr_t y2,
+                                 int64_t ldy2, uintptr_t pw1, uintptr_t pw2, uintptr_t post_w, float mult, uintptr_t extra,
+                                 uintptr_t next_w, float off, float eps, uintptr_t out, bool out_f32, int T, int W,
+                                 uintptr_t st) {
+    if ((y && ldy < W) || (y2 && ldy2 < W)) throw std::invalid_argument("post_norm_residual: row stride below the width");
+    int rc = xgm::post_norm_residual(P<float>(x), P<const void>(y), y_f32, ldy, P<const float>(y_bias), P<const void>(y2),
+                                     ldy2, P<const float>(pw1), P<const float>(pw2), P<const float>(post_w), mult,
+                                     P<const float>(extra), P<const float>(next_w), off, eps, P<void>(out), out_f32, T, W,
+                                     S(st));
+    check(rc, "post_norm_residual");
+  });
+  m.def("relu2", [](uintptr_t in, bool f32, uintptr_t bias, uintptr_t out, int64_t n, int cols, uintptr_t st) {
+    if (cols < 1 || n % cols) throw std::invalid_argument("relu2: the element count must be whole rows");
+    xgm::relu2(P<const void>(in), f32, P<const float>(bias), P<void>(out), n, cols, S(st));
+    check(0, "relu2");
+  });
+  m.def("lower_bound_gates", [](uintptr_t proj, bool f32, int64_t ld, int off_q, int off_f, int n, uintptr_t f_bias,
+                                uintptr_t lower, uintptr_t q, uintptr_t f, int T, uintptr_t st) {
+    if (n < 1 || off_q < 0 || off_f < 0 || ld < off_q + n || ld < off_f + n)
+      throw std::invalid_argument("lower_bound_gates: columns outside the row");
+    xgm::lower_bound_gates(P<const void>(proj), f32, ld, off_q, off_f, n, P<const float>(f_bias), P<const float>(lower),
+                           P<float>(q), P<float>(f), T, S(st));
+    check(0, "lower_bound_gates");
+  });
+  m.def("gated_linear_scan", [](uintptr_t q, uintptr_t f, uintptr_t k, uintptr_t v, bool v_f32, int64_t ld_v,
+                                uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t o, int ns, int H,
+                                int dk, int dv, uintptr_t st) {
+    if (H < 1 || dv < 1 || ld_v < (int64_t)H * dv) throw std::invalid_argument("gated_linear_scan: inconsistent sizes");
+    int rc = xgm::gated_linear_scan(P<const float>(q), P<const float>(f), P<const float>(k), P<const void>(v), v_f32, ld_v,
+                                    P<float>(state), P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
+                                    P<float>(o), ns, H, dk, dv, S(st));
+    check(rc, "gated_linear_scan");
   });
   m.def("ssm_scan", [](uintptr_t xbc, bool f32, int64_t ld_x, uintptr_t dt, int64_t ld_dt, uintptr_t dt_bias,
                        uintptr_t A_log, uintptr_t D, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,
@@ -127,11 +199,12 @@ PYBIND11_MODULE(_mixers, m) {
                            P<const int32_t>(sl), P<const int32_t>(slots), P<float>(y), ns, H, G, N, Pd, S(st));
     check(rc, "ssm_scan");
   });
-  m.def("gated_group_norm", [](uintptr_t y, uintptr_t z, bool f32, int64_t ld_z, uintptr_t w, float eps, uintptr_t out,
-                               int T, int inner, int ng, uintptr_t st) {
-    if (ng < 1 || inner % ng) throw std::invalid_argument("gated_group_norm: the parts must divide the row");
-    xgm::gated_group_norm(P<const float>(y), P<const void>(z), f32, ld_z, P<const float>(w), eps, P<void>(out), T, inner,
-                          ng, S(st));
+  m.def("gated_group_norm", [](uintptr_t y, uintptr_t z, bool f32, int64_t ld_z, uintptr_t w, int wn, float eps,
+                               uintptr_t out, int T, int inner, int ng, uintptr_t st) {
+    if (ng < 1 || inner % ng || wn < 1 || inner % wn)
+      throw std::invalid_argument("gated_group_norm: the parts and the weight's period must divide the row");
+    xgm::gated_group_norm(P<const float>(y), P<const void>(z), f32, ld_z, P<const float>(w), wn, eps, P<void>(out), T,
+                          inner, ng, S(st));
     check(0, "gated_group_norm");
   });
   m.def("glu_act", [](uintptr_t in, bool f32, int64_t ld, uintptr_t out, int T, int F, int kind, float limit, float alpha,
