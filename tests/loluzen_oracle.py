@@ -100,8 +100,9 @@ def conv_rope_attention(Wt, pre, m, h, eps):
     v = shifted_conv(h @ Wt[pre + "v"].T, Wt[pre + "v.conv"]).reshape(T, G, dv)
     q = unit_rms(q, eps) * Wt[pre + "q.norm"]
     k = unit_rms(k, eps) * Wt[pre + "k.norm"]
-    fr = rot_frequencies(m["rot"])
-    q, k = rotate_pairs(q, fr, int(m["rot"]["dims"])), rotate_pairs(k, fr, int(m["rot"]["dims"]))
+    if m.get("rot") and int(m["rot"]["dims"]) > 0:
+        fr = rot_frequencies(m["rot"])
+        q, k = rotate_pairs(q, fr, int(m["rot"]["dims"])), rotate_pairs(k, fr, int(m["rot"]["dims"]))
     P = causal_weights(q, k, float(m["scale"]))
     gate = torch.sigmoid(h @ Wt[pre + "g"].T)                            # [T, H]
     o = torch.stack([P[hd] @ v[:, hd // (H // G)] for hd in range(H)], 1) * gate[:, :, None]
@@ -203,3 +204,75 @@ def forward(cfg, Wt, tokens, residuals=None):
         if residuals is not None:
             residuals.append(x.clone())
     return N(x, "final.norm") @ Wt["head"].T
+
+
+# ------------------------------------------------------------------------------ test models
+def random_weights(config, seed=0):
+    """Random weights of a configuration, rounded to bfloat16 (what a checkpoint stores)."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = config["width"], config["vocab"]
+    out = {}
+
+    def mat(name, o, i, gain=1.0):
+        out[name] = torch.randn(o, i, generator=g) * gain / math.sqrt(i)
+
+    def vec(name, n, std, mean=0.0):
+        out[name] = torch.randn(n, generator=g) * std + mean
+    out["embed"] = torch.randn(V, W, generator=g) * 0.5
+    mat("head", V, W)
+    vec("final.norm", W, 0.2)
+    for n, layer in enumerate(config["layers"]):
+        pre, m = f"l{n}.", layer["mixer"]
+        vec(pre + "norm1", W, 0.2)
+        vec(pre + "norm1b", W, 0.2)
+        if layer["type"] == "attention":
+            H, G, dk, dv, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+            for nm, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv)):
+                mat(pre + "mix." + nm, rows, W, 2.0)
+                out[pre + "mix." + nm + ".conv"] = torch.randn(rows, taps, generator=g) * 0.5 + 1.0 / taps
+            vec(pre + "mix.q.norm", dk, 0.3, 1.5)
+            vec(pre + "mix.k.norm", dk, 0.3, 1.5)
+            mat(pre + "mix.g", H, W, 2.0)
+            mat(pre + "mix.o", W, H * dv)
+        else:
+            a, r = m["left"], m["right"]
+            H, G, dk, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            for nm, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv)):
+                mat(pre + "mix.left." + nm, rows, W, 2.0)
+                vec(pre + "mix.left." + nm + ".b", rows, 0.3)
+            out[pre + "mix.left.r1"] = torch.rand(H, generator=g) * 2.0
+            out[pre + "mix.left.r2"] = torch.rand(H, generator=g) * 3.0 + 0.05
+            out[pre + "mix.left.talk"] = torch.eye(H) * 0.7 + torch.randn(H, H, generator=g) * 0.4
+            mat(pre + "mix.left.g", H, W, 2.0)
+            mat(pre + "mix.left.o", W, H * dv)
+            n_, Hr = r["heads"] * r["dim"], r["heads"]
+            mat(pre + "mix.right.q", n_, W, 2.0)
+            mat(pre + "mix.right.f", n_, W, 2.0)
+            vec(pre + "mix.right.f.b", n_, 0.5, 1.0)
+            out[pre + "mix.right.lower"] = torch.rand(n_, generator=g) * 0.95
+            mat(pre + "mix.right.v", Hr * r["vdim"], W, 2.0)
+            vec(pre + "mix.right.norm", r["vdim"], 0.3, 1.0)
+            mat(pre + "mix.right.o", W, Hr * r["vdim"])
+            vec(pre + "mix.left.out", W, 0.3, 1.0)
+            vec(pre + "mix.right.out", W, 0.3, 1.0)
+        mlp = layer.get("mlp")
+        if mlp is None:
+            continue
+        vec(pre + "norm2", W, 0.2)
+        vec(pre + "norm2b", W, 0.2)
+        mat(pre + "mlp.up", mlp["ff"], W, 1.5)
+        vec(pre + "mlp.up.b", mlp["ff"], 0.3)
+        mat(pre + "mlp.down", W, mlp["ff"])
+        vec(pre + "mlp.down.b", W, 0.3)
+    return {k: v.to(torch.bfloat16).to(F64) for k, v in out.items()}
+
+
+def write_checkpoint(path, config, Wt):
+    import json
+    import os
+
+    from safetensors.torch import save_file
+    os.makedirs(path, exist_ok=True)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in Wt.items()}, os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(config, f)
