@@ -54,7 +54,7 @@ def config_a():
 def config_b():
     """One head; one tap (no carried convolution inputs); no rotation; no loop; factors of one; a loop of one
     pass would be the same model."""
-    a1 = {"heads": 1, "kv_heads": 1, "dim": 32, "vdim": 32, "scale": 1.0, "conv": 1}
+    a1 = {"heads": 1, "kv_heads": 1, "dim": 32, "vdim": 32, "scale": 0.2, "conv": 1}
     a2 = {"heads": 4, "kv_heads": 1, "dim": 16, "vdim": 8, "scale": 0.5, "conv": 3,
           "rot": {"base": 10.0, "dims": 2, "scaling": {"factor": 2.0, "low": 1.0, "high": 2.0, "original": 8}}}
     par = {"left": {"heads": 1, "kv_heads": 1, "dim": 16, "vdim": 16, "scale": 0.25},
