@@ -79,6 +79,12 @@ def parse():
                          "batch, --steps, --warmup, --dofivik-prompts, --dofivik-context apply)")
     ap.add_argument("--vizonex-sizes", default="1b-class,8b-class")
     ap.add_argument("--vizonex-only", default=None, choices=["vizonex", "mixtral", "llama"])
+    ap.add_argument("--loluzen", action="store_true",
+                    help="instead of the headline: prefill and decode tokens/s of Loluzen beside a Llama of equal layer "
+                         "sizes (bench/loluzen_bench.py; --prompt-len, --concurrency = decode batch, --steps, --warmup, "
+                         "--dofivik-prompts, --dofivik-context apply)")
+    ap.add_argument("--loluzen-sizes", default="1b-class,8b-class")
+    ap.add_argument("--loluzen-only", default=None, choices=["loluzen", "llama"])
     return ap.parse_args()
 
 
@@ -173,11 +179,11 @@ def preflight(st, world: int, tp: int, dev, eng) -> dict:
 
 def main():
     a = parse()
-    if a.dofivik or a.vizonex:
+    if a.dofivik or a.vizonex or a.loluzen:
         import importlib.util
         here = os.path.dirname(os.path.abspath(__file__))
         sys.path.insert(0, here)
-        which = "dofivik_bench" if a.dofivik else "vizonex_bench"
+        which = "dofivik_bench" if a.dofivik else "vizonex_bench" if a.vizonex else "loluzen_bench"
         spec = importlib.util.spec_from_file_location(which, os.path.join(here, "bench", which + ".py"))
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
