@@ -190,8 +190,16 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
 // operand (V^T) is a transposed LDS read of the staged V rows.
 constexpr int kKT = 64;
 
-template <int NKK_MAX, int NMT_MAX>
-__global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
+__device__ __forceinline__ float exp2_fast(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_exp2f(x);
+#else
+  return exp2f(x);
+#endif
+}
+
+template <int NKK_MAX, int NMT_MAX, int NW>
+__global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int32_t* __restrict__ block_tables, int bt_width, int bs, const int32_t* __restrict__ qsl,
     const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, const float* __restrict__ temp,
@@ -216,8 +224,9 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
     return;
   }
   // prompt portions: slots = 16 tokens of one head; single-token steps (head_slots): slots = 16 heads of the token
-  const int tpb = head_slots ? 1 : 4 / RH;  // token tiles per workgroup
-  const int t0 = head_slots ? 0 : blockIdx.x * 16 * tpb;
+  const int tpb = head_slots ? 1 : NW / RH;  // token tiles per workgroup
+  // late token tiles see the most keys: they are dispatched first
+  const int t0 = head_slots ? 0 : ((int)gridDim.x - 1 - (int)blockIdx.x) * 16 * tpb;
   if (t0 >= qn) return;
   const int hblocks = (rep + RH - 1) / RH;
   const int g = head_slots ? blockIdx.y : blockIdx.y / hblocks, hb = blockIdx.y % hblocks;
@@ -231,6 +240,11 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
   const int ctx = seq_lens[s] - qn;
   const int pos_q = ctx + min(tok, qn - 1);
   const int lo_q = first_visible(mask, size, pos_q);
+  // a key tile [k0, k0 + 63] needs no per-key test when every slot of the wave sees all of it (wave-uniform)
+  const int tw = head_slots ? 0 : t0 + (wave / RH) * 16;               // the wave's first token
+  const bool slots_full = head_slots || tw + 16 <= qn;
+  const int pos_w0 = ctx + min(tw, qn - 1);
+  const int lo_w1 = first_visible(mask, size, ctx + min(head_slots ? 0 : tw + 15, qn - 1));
   const int nkk = dk / 32, nmt = dv / 16;
   // keys any slot of this workgroup can see
   int kmin = first_visible(mask, size, ctx + t0);
@@ -251,19 +265,21 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
     if (kk < nkk && valid) v = xgk::ld16(q + ((int64_t)(q0 + tok) * H + head) * dk + kk * 32 + kg * 8);
     qf[kk] = xgk::as_frag(v);
   }
-  const float sc_h = scale * (temp ? temp[head] : 1.f);
+  // scores are kept in units of ln 2 (exp2 is one instruction): score * log2(e)
+  constexpr float kLog2e = 1.4426950408889634f;
+  const float sc_h = scale * (temp ? temp[head] : 1.f) * kLog2e;
   xgk::f32x4_t o[NMT_MAX];
 #pragma unroll
   for (int mt = 0; mt < NMT_MAX; ++mt) o[mt] = xgk::f32x4_t{0.f, 0.f, 0.f, 0.f};
   // the sink starts the running softmax: weight exp(sink - m) = 1 with no value behind it
   const bool with_sink = sink && (nsplit == 1 || blockIdx.x == 0);  // the sink enters the first share only
-  float m = with_sink ? sink[head] : -INFINITY, l = with_sink ? 1.f : 0.f;
+  float m = with_sink ? sink[head] * kLog2e : -INFINITY, l = with_sink ? 1.f : 0.f;
 
-  // staging: thread -> (row = tid / 4, 16-byte chunks tid % 4, + 4, ..) of the K row and of the V row. The next
+  // staging: thread -> (row = tid / NW, 16-byte chunks tid % NW, + NW, ..) of the K row and of the V row. The next
   // tile's rows are loaded into registers before the current tile's products and stored after them.
-  const int srow = threadIdx.x >> 2, squad = threadIdx.x & 3;
-  constexpr int NVC = (NMT_MAX + 1) / 2;
-  uint4 sk[NKK_MAX], sv[NVC];
+  const int srow = threadIdx.x / NW, squad = threadIdx.x % NW;
+  constexpr int NKC = (NKK_MAX * 4 + NW - 1) / NW, NVC = (NMT_MAX * 2 + NW - 1) / NW;
+  uint4 sk[NKC], sv[NVC];
   auto fetch = [&](int k0) {
     const int kabs = k0 + srow;
     const bool ok = kabs <= pos_last;
@@ -271,25 +287,25 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
     const bf16* ks = kcache + (row * G + g) * dk;
     const bf16* vs = vcache + row * G * dv_head + voff;
 #pragma unroll
-    for (int it = 0; it < NKK_MAX; ++it) {
-      const int ch = squad + 4 * it;
+    for (int it = 0; it < NKC; ++it) {
+      const int ch = squad + NW * it;
       sk[it] = (ok && ch * 8 < dk) ? xgk::ld16(ks + ch * 8) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int it = 0; it < NVC; ++it) {
-      const int ch = squad + 4 * it;
+      const int ch = squad + NW * it;
       sv[it] = (ok && ch * 8 < dv) ? xgk::ld16(vs + ch * 8) : make_uint4(0, 0, 0, 0);
     }
   };
   auto commit = [&]() {
 #pragma unroll
-    for (int it = 0; it < NKK_MAX; ++it) {
-      const int ch = squad + 4 * it;
+    for (int it = 0; it < NKC; ++it) {
+      const int ch = squad + NW * it;
       if (ch * 8 < dk) xgk::st16(ktile + srow * LDK + ch * 8, sk[it]);
     }
 #pragma unroll
     for (int it = 0; it < NVC; ++it) {
-      const int ch = squad + 4 * it;
+      const int ch = squad + NW * it;
       if (ch * 8 < dv) xgk::st16(vtile + srow * LDV + ch * 8, sv[it]);
     }
   };
@@ -311,27 +327,29 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
                                       sacc[n]);
     }
     float mx = -INFINITY;
+    const bool full = slots_full && k0 + kKT - 1 <= pos_w0 && k0 >= lo_w1;
 #pragma unroll
     for (int n = 0; n < 4; ++n)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int kabs = k0 + n * 16 + kg * 4 + r;
         float v = sacc[n][r] * sc_h;
-        if (r1) v -= pen1 * __logf(1.f + pen2 * (float)max(pos_q - kabs, 0));
-        if (!valid || kabs > pos_q || kabs < lo_q) v = -INFINITY;
+        // r1 ln(1 + r2 d) in units of ln 2 is r1 log2(1 + r2 d)
+        if (r1) v -= pen1 * __log2f(1.f + pen2 * (float)max(pos_q - kabs, 0));
+        if (!full && (!valid || kabs > pos_q || kabs < lo_q)) v = -INFINITY;
         sacc[n][r] = v;
         mx = fmaxf(mx, v);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
-    const float alpha = (m_new == -INFINITY || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : __expf(m - m_new);
+    const float alpha = (m_new == -INFINITY || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : exp2_fast(m - m_new);
     float rs = 0.f;
 #pragma unroll
     for (int n = 0; n < 4; ++n)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = m_new == -INFINITY ? 0.f : __expf(sacc[n][r] - m_new);
+        const float p = m_new == -INFINITY ? 0.f : exp2_fast(sacc[n][r] - m_new);
         sacc[n][r] = p;
         rs += p;
       }
@@ -389,7 +407,7 @@ __global__ __launch_bounds__(256) void masked_attention_mfma_kernel(
   }
 }
 
-// merge the key shares of a single-token step: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s
+// merge the key shares of a single-token step: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s (m in units of ln 2)
 __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                 const int32_t* __restrict__ slots, bf16* __restrict__ out, int Ttot, int H,
                                                 int dv, int nsplit, const bf16* __restrict__ gate, int64_t ld_gate) {
@@ -401,7 +419,7 @@ __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o
   for (int sp = 0; sp < nsplit; ++sp) {
     const int64_t row = ((int64_t)sp * Ttot + t) * H + h;
     const float ms = part_ml[2 * row];
-    if (ms != -INFINITY) L += __expf(ms - M) * part_ml[2 * row + 1];
+    if (ms != -INFINITY) L += exp2_fast(ms - M) * part_ml[2 * row + 1];
   }
   float inv = L > 0.f ? 1.f / L : 0.f;
   if (gate) inv *= sigmoidf(bf2f(gate[(int64_t)t * ld_gate + h]));
@@ -410,7 +428,7 @@ __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o
     for (int sp = 0; sp < nsplit; ++sp) {
       const int64_t row = ((int64_t)sp * Ttot + t) * H + h;
       const float ms = part_ml[2 * row];
-      if (ms != -INFINITY) acc += __expf(ms - M) * part_o[row * dv + d];
+      if (ms != -INFINITY) acc += exp2_fast(ms - M) * part_o[row * dv + d];
     }
     out[((int64_t)t * H + h) * dv + d] = f2bf(acc * inv);
   }
@@ -426,6 +444,27 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(const T* __restrict__ o_a
   const int t = blockIdx.x;
   const int rep = H / G;
   const T* row = o_all + (int64_t)t * H * G * dv;
+  if ((dv & 3) == 0) {  // four value columns per thread
+    for (int e = threadIdx.x; e < H * dv / 4; e += blockDim.x) {
+      const int h = e / (dv / 4), d = 4 * (e % (dv / 4));
+      const int c = h / rep;
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int g = 0; g < H; ++g) {
+        float v[4];
+        ld4(row + ((int64_t)g * G + c) * dv + d, v);
+        const float w = talk[h * H + g];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += w * v[i];
+      }
+      if (gate) {
+        const float sg = sigmoidf(ldf(gate + (int64_t)t * ld_gate + h));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= sg;
+      }
+      st4(out + (int64_t)t * H * dv + h * dv + d, acc);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < H * dv; e += blockDim.x) {
     const int h = e / dv, d = e % dv;
     const int c = h / rep;
@@ -536,7 +575,7 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
                           int bs, const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, const float* temp,
                           const float* sink, void* out, int T_, int ns, int max_q, int H, int G, int dk, int dv_head,
                           int mask, int size, float scale, int nsplit, float* part_o, float* part_ml, const void* gate,
-                          int64_t ld_gate, const float* r1, const float* r2, int vmode, hipStream_t st) {
+                          int64_t ld_gate, const float* r1, const float* r2, int vmode, int nw_hint, hipStream_t st) {
   if (T_ <= 0 || ns <= 0 || max_q <= 0) return 0;
   const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
   if (G <= 0 || H % G != 0 || dk % 32 != 0 || dv % 16 != 0 || dk > 128 || dv > 256 || mask < 0 || mask > 2 ||
@@ -544,21 +583,31 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
     return -1;
   const int rep = H / G;
   const int RH = rep >= 4 ? 4 : rep >= 2 ? 2 : 1;
-  const int tpb = 4 / RH;
   // a step of single tokens: one workgroup per (sequence, key/value head), its query heads as the slots
   const int head_slots = (max_q == 1 && T_ == ns) ? 1 : 0;
   if (head_slots && rep > 64) return -3;
+  // waves per workgroup: 4 for single tokens and short portions, 8 for long portions (twice the token tiles of the same
+  // heads on every staged key tile; 16 waves measured slower: the early tiles of a 64-token span idle at the late keys)
+  int nw = (head_slots || max_q <= 32) ? 4 : 8;
+  if (!head_slots && (nw_hint == 4 || nw_hint == 8 || (nw_hint == 16 && dv <= 128))) nw = nw_hint;
+  const int tpb = nw / RH;
   dim3 grid((max_q + 16 * tpb - 1) / (16 * tpb), G * ((rep + RH - 1) / RH), ns);
   if (!head_slots || nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) nsplit = 1;
   if (head_slots) grid = dim3(nsplit, G, ns);
   const size_t lds = (size_t)kKT * (dk + 8 + dv + 8) * sizeof(uint16_t);
+#define XGM_MK(NKK, NMT, NW)                                                                                          \
+  masked_attention_mfma_kernel<NKK, NMT, NW><<<grid, 64 * NW, lds, st>>>(                                             \
+      (const bf16*)q, (const bf16*)kcache, (const bf16*)vcache, block_tables, bt_width, bs, qsl, seq_lens, slots, temp, \
+      sink, (bf16*)out, H, G, dk, dv_head, mask, size, scale, RH, head_slots, part_o, part_ml, T_, (const bf16*)gate,  \
+      ld_gate, r1, r2, vmode);
 #define XGM_MM(NKK, NMT)                                                                                              \
-  masked_attention_mfma_kernel<NKK, NMT><<<grid, 256, lds, st>>>((const bf16*)q, (const bf16*)kcache,                 \
-                                                                 (const bf16*)vcache, block_tables, bt_width, bs, qsl, \
-                                                                 seq_lens, slots, temp, sink, (bf16*)out, H, G, dk,    \
-                                                                 dv_head, mask, size, scale, RH, head_slots, part_o,   \
-                                                                 part_ml, T_, (const bf16*)gate, ld_gate, r1, r2,      \
-                                                                 vmode);                                               \
+  if (nw == 16 && NMT <= 8) {                                                                                         \
+    XGM_MK(NKK, NMT, (NMT <= 8 ? 16 : 8))                                                                             \
+  } else if (nw >= 8) {                                                                                               \
+    XGM_MK(NKK, NMT, 8)                                                                                               \
+  } else {                                                                                                            \
+    XGM_MK(NKK, NMT, 4)                                                                                               \
+  }                                                                                                                   \
   if (nsplit > 1)                                                                                                     \
     masked_attention_combine_kernel<<<dim3(T_, H), 64, 0, st>>>(part_o, part_ml, slots, (bf16*)out, T_, H, dv, nsplit, \
                                                                 (const bf16*)gate, ld_gate);                          \
@@ -568,6 +617,7 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
   if (dk <= 128 && dv <= 256) { XGM_MM(4, 16) }
   return -2;
 #undef XGM_MM
+#undef XGM_MK
 }
 
 void talk_mix(const void* o_all, bool f32, const float* talk, const void* gate, int64_t ld_gate, void* out, int T_, int H,

@@ -6,6 +6,8 @@
 //   gated_linear_scan  per head, state S [dk x dv] fp32 per (slot, head):
 //                        S_t = diag(f_t) S_(t-1) + k_t v_t^T        (k_t = 1 - f_t when k == nullptr)
 //                        o_t = S_t^T q_t
+//                      q / f / k are fp32 tensors, or (raw form) q and f are taken straight from the fused
+//                      projection row and pass silu / the lower-bounded sigmoid while they are staged
 //
 // One workgroup = (sequence, head, 64 state columns), NW waves: lane p owns column p, wave w owns rows
 // [w * NI, (w + 1) * NI) of it in registers. f / k / q / v of TT tokens at a time are staged in LDS (two buffers:
@@ -32,14 +34,20 @@ __global__ void lower_bound_gates_kernel(const T* __restrict__ proj, int64_t ld,
 
 constexpr int kGlaCols = 64;   // state columns per workgroup
 
-template <typename T, int NI, int TT, int NW>
+// RAW: q and f are read as columns [off_q, off_q + H dk) / [off_f, ..) of the activation rows `raw` and go
+// through silu / the lower-bounded sigmoid while they are staged (no pass of their own, half the bytes), and the
+// write strength is 1 - f. Otherwise q, f (and k, or 1 - f when k == nullptr) are fp32 tensors [T, H dk].
+template <typename T, int NI, int TT, int NW, bool RAW>
 __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
-    const float* __restrict__ q, const float* __restrict__ f, const float* __restrict__ k, const T* __restrict__ v,
-    int64_t ld_v, float* __restrict__ state, const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens,
-    const int32_t* __restrict__ slots, float* __restrict__ o, int H, int dk, int dv) {
+    const float* __restrict__ q, const float* __restrict__ f, const float* __restrict__ k, const T* __restrict__ raw,
+    int64_t ld_raw, int off_q, int off_f, const float* __restrict__ f_bias, const float* __restrict__ lower,
+    const T* __restrict__ v, int64_t ld_v, float* __restrict__ state, const int32_t* __restrict__ qsl,
+    const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, float* __restrict__ o, int H, int dk,
+    int dv) {
   constexpr int NB = NW * NI;                // padded state rows
   constexpr int NTH = 64 * NW;
-  constexpr int ROW = 3 * NB + kGlaCols;     // staged floats per token: [f | k | q | v]
+  constexpr int NQ = RAW ? 2 : 3;            // staged row blocks: [f | q | (k)]
+  constexpr int ROW = NQ * NB + kGlaCols;    // staged floats per token: [f | q | (k) | v]
   constexpr int PER = (TT * ROW + NTH - 1) / NTH;
   __shared__ __attribute__((aligned(16))) float stage[2][TT][ROW];
   __shared__ float opart[TT][NW][kGlaCols];
@@ -68,16 +76,21 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
       float val = 0.f;
       if (tt < nt) {
         const int64_t tok = q0 + t0 + tt;
-        if (c < NB) {
-          if (c < dk) val = f[tok * nqk + h * dk + c];
-        } else if (c < 2 * NB) {
-          const int cc = c - NB;
-          if (cc < dk) val = k ? k[tok * nqk + h * dk + cc] : 1.f - f[tok * nqk + h * dk + cc];
-        } else if (c < 3 * NB) {
-          const int cc = c - 2 * NB;
-          if (cc < dk) val = q[tok * nqk + h * dk + cc];
-        } else if (p0 + c - 3 * NB < dv) {
-          val = ldf(v + tok * ld_v + h * dv + p0 + c - 3 * NB);
+        const int blk = c / NB, cc = c % NB;
+        if (blk < NQ) {
+          if (cc < dk) {
+            if (RAW) {
+              val = ldf(raw + tok * ld_raw + (blk == 0 ? off_f : off_q) + h * dk + cc);
+            } else if (blk == 0) {
+              val = f[tok * nqk + h * dk + cc];
+            } else if (blk == 1) {
+              val = q[tok * nqk + h * dk + cc];
+            } else {
+              val = k ? k[tok * nqk + h * dk + cc] : 1.f - f[tok * nqk + h * dk + cc];
+            }
+          }
+        } else if (p0 + c - NQ * NB < dv) {
+          val = ldf(v + tok * ld_v + h * dv + p0 + c - NQ * NB);
         }
       }
       pre[j] = val;
@@ -87,7 +100,21 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int e = threadIdx.x + NTH * j;
-      if (e < TT * ROW) (&stage[buf][0][0])[e] = pre[j];
+      if (e < TT * ROW) {
+        float val = pre[j];
+        if (RAW) {
+          const int c = e % ROW, blk = c / NB, cc = c % NB;
+          if (blk < NQ && cc < dk) {
+            if (blk == 0) {
+              const float l = lower[h * dk + cc];
+              val = l + (1.f - l) * sigmoidf(val + (f_bias ? f_bias[h * dk + cc] : 0.f));
+            } else {
+              val = siluf(val);
+            }
+          }
+        }
+        (&stage[buf][0][0])[e] = val;
+      }
     }
   };
   fetch(0);
@@ -98,18 +125,25 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
     const int nt = min(TT, qn - t0);
     const bool more = t0 + TT < qn;
     if (more) fetch(t0 + TT);
-    for (int tt = 0; tt < nt; ++tt) {
+    auto step = [&](int tt) {
       const float* fr = &stage[buf][tt][wave * NI];
-      const float* kr = &stage[buf][tt][NB + wave * NI];
-      const float* qr = &stage[buf][tt][2 * NB + wave * NI];
-      const float vv = stage[buf][tt][3 * NB + lane];
+      const float* qr = &stage[buf][tt][NB + wave * NI];
+      const float* kr = &stage[buf][tt][(NQ - 1) * NB + wave * NI];   // RAW: unused
+      const float vv = stage[buf][tt][NQ * NB + lane];
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        S[i] = fr[i] * S[i] + kr[i] * vv;
-        acc += S[i] * qr[i];
+        // k = 1 - f:  f S + (1 - f) v = v + f (S - v), one operation less per element
+        S[i] = RAW ? fmaf(fr[i], S[i] - vv, vv) : fmaf(fr[i], S[i], kr[i] * vv);
+        acc = fmaf(S[i], qr[i], acc);
       }
       opart[tt][wave][lane] = acc;
+    };
+    if (nt == TT) {  // whole tile: a fixed trip count lets the LDS reads of several steps be in flight together
+#pragma unroll 4
+      for (int tt = 0; tt < TT; ++tt) step(tt);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) step(tt);
     }
     __syncthreads();
     for (int e = threadIdx.x; e < nt * kGlaCols; e += NTH) {
@@ -142,23 +176,32 @@ void lower_bound_gates(const void* proj, bool f32, int64_t ld, int off_q, int of
                           (const T*)proj, ld, off_q, off_f, n, f_bias, lower, q, f, total);)
 }
 
-int gated_linear_scan(const float* q, const float* f, const float* k, const void* v, bool v_f32, int64_t ld_v, float* state,
+int gated_linear_scan(const float* q, const float* f, const float* k, const void* raw, int64_t ld_raw, int off_q, int off_f,
+                      const float* f_bias, const float* lower, const void* v, bool v_f32, int64_t ld_v, float* state,
                       const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, float* o, int ns, int H, int dk,
                       int dv, hipStream_t st) {
   if (ns <= 0) return 0;
-  if (H <= 0 || dk < 1 || dk > 256 || dv < 1) return -1;
+  if (H <= 0 || dk < 1 || dk > 256 || dv < 1 || (raw ? !lower : (!q || !f))) return -1;
   dim3 grid(ns, H, (dv + kGlaCols - 1) / kGlaCols);
-#define XGM_GL(NI, TT, NW)                                                                                              \
-  XGM_DISPATCH_T(v_f32, gated_linear_scan_kernel<T, NI, TT, NW><<<grid, 64 * NW, 0, st>>>(q, f, k, (const T*)v, ld_v, state, \
-                                                                                          qsl, seq_lens, slots, o, H, dk, \
-                                                                                          dv);)                         \
+#define XGM_GL2(NI, TT, NW, RAW)                                                                                       \
+  XGM_DISPATCH_T(v_f32, gated_linear_scan_kernel<T, NI, TT, NW, RAW><<<grid, 64 * NW, 0, st>>>(                         \
+                            q, f, k, (const T*)raw, ld_raw, off_q, off_f, f_bias, lower, (const T*)v, ld_v, state, qsl, \
+                            seq_lens, slots, o, H, dk, dv);)
+  // tokens per staged tile: the raw form stages two row blocks instead of three and takes longer tiles
+#define XGM_GL(NI, TT, TTR, NW)           \
+  if (raw) {                              \
+    XGM_GL2(NI, TTR, NW, true)            \
+  } else {                                \
+    XGM_GL2(NI, TT, NW, false)            \
+  }                                       \
   return 0;
-  if (dk <= 16) { XGM_GL(4, 16, 4) }
-  if (dk <= 32) { XGM_GL(8, 16, 4) }
-  if (dk <= 64) { XGM_GL(8, 8, 8) }
-  if (dk <= 128) { XGM_GL(16, 8, 8) }
-  XGM_GL(32, 4, 8)
+  if (dk <= 16) { XGM_GL(4, 16, 32, 4) }
+  if (dk <= 32) { XGM_GL(8, 16, 32, 4) }
+  if (dk <= 64) { XGM_GL(8, 8, 16, 8) }
+  if (dk <= 128) { XGM_GL(16, 8, 8, 8) }
+  XGM_GL(32, 4, 4, 8)
 #undef XGM_GL
+#undef XGM_GL2
 }
 
 }  // namespace xgm

@@ -23,7 +23,8 @@ int masked_attention(const void*, bool, const void*, const void*, const int32_t*
                      const void*, int64_t, const float*, const float*, int, hipStream_t);
 int masked_attention_mfma(const void*, const void*, const void*, const int32_t*, int, int, const int32_t*, const int32_t*,
                           const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, int, int,
-                          float, int, float*, float*, const void*, int64_t, const float*, const float*, int, hipStream_t);
+                          float, int, float*, float*, const void*, int64_t, const float*, const float*, int, int,
+                          hipStream_t);
 void talk_mix(const void*, bool, const float*, const void*, int64_t, void*, int, int, int, int, hipStream_t);
 void head_norm_rope_cache(const void*, bool, int64_t, int, int, int, int, const float*, const float*, float, const float*,
                           int, int, const int32_t*, const int32_t*, void*, void*, void*, bool, int, hipStream_t);
@@ -32,8 +33,9 @@ int post_norm_residual(float*, const void*, bool, int64_t, const float*, const v
 void relu2(const void*, bool, const float*, void*, int64_t, int, hipStream_t);
 void lower_bound_gates(const void*, bool, int64_t, int, int, int, const float*, const float*, float*, float*, int,
                        hipStream_t);
-int gated_linear_scan(const float*, const float*, const float*, const void*, bool, int64_t, float*, const int32_t*,
-                      const int32_t*, const int32_t*, float*, int, int, int, int, hipStream_t);
+int gated_linear_scan(const float*, const float*, const float*, const void*, int64_t, int, int, const float*, const float*,
+                      const void*, bool, int64_t, float*, const int32_t*, const int32_t*, const int32_t*, float*, int, int,
+                      int, int, hipStream_t);
 int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, const float*, const float*, float*,
              const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, int, int, hipStream_t);
 void gated_group_norm(const float*, const void*, bool, int64_t, const float*, int, float, void*, int, int, int,
@@ -124,7 +126,7 @@ PYBIND11_MODULE(_mixers, m) {
                                     uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t temp, uintptr_t sink,
                                     uintptr_t out, int T, int ns, int max_q, int H, int G, int dk, int dv, int mask,
                                     int size, float scale, int nsplit, uintptr_t part_o, uintptr_t part_ml,
-                                    uintptr_t gate, int64_t ld_gate, uintptr_t r1, uintptr_t r2, int vmode,
+                                    uintptr_t gate, int64_t ld_gate, uintptr_t r1, uintptr_t r2, int vmode, int nw_hint,
                                     uintptr_t st) {
     if (bs < 1 || bt_width < 1 || nsplit < 1 || (gate && ld_gate < H))
       throw std::invalid_argument("masked_attention_mfma: inconsistent sizes");
@@ -133,7 +135,7 @@ PYBIND11_MODULE(_mixers, m) {
                                         P<const float>(temp), P<const float>(sink), P<void>(out), T, ns, max_q, H, G, dk,
                                         dv, mask, size, scale, nsplit, P<float>(part_o), P<float>(part_ml),
                                         P<const void>(gate), ld_gate, P<const float>(r1), P<const float>(r2), vmode,
-                                        S(st));
+                                        nw_hint, S(st));
     check(rc, "masked_attention_mfma");
   });
   m.def("talk_mix", [](uintptr_t o_all, bool f32, uintptr_t talk, uintptr_t gate, int64_t ld_gate, uintptr_t out, int T,
@@ -180,13 +182,17 @@ PYBIND11_MODULE(_mixers, m) {
                            P<float>(q), P<float>(f), T, S(st));
     check(0, "lower_bound_gates");
   });
-  m.def("gated_linear_scan", [](uintptr_t q, uintptr_t f, uintptr_t k, uintptr_t v, bool v_f32, int64_t ld_v,
-                                uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t o, int ns, int H,
-                                int dk, int dv, uintptr_t st) {
-    if (H < 1 || dv < 1 || ld_v < (int64_t)H * dv) throw std::invalid_argument("gated_linear_scan: inconsistent sizes");
-    int rc = xgm::gated_linear_scan(P<const float>(q), P<const float>(f), P<const float>(k), P<const void>(v), v_f32, ld_v,
-                                    P<float>(state), P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
-                                    P<float>(o), ns, H, dk, dv, S(st));
+  m.def("gated_linear_scan", [](uintptr_t q, uintptr_t f, uintptr_t k, uintptr_t raw, int64_t ld_raw, int off_q, int off_f,
+                                uintptr_t f_bias, uintptr_t lower, uintptr_t v, bool v_f32, int64_t ld_v, uintptr_t state,
+                                uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t o, int ns, int H, int dk, int dv,
+                                uintptr_t st) {
+    if (H < 1 || dv < 1 || dk < 1 || ld_v < (int64_t)H * dv ||
+        (raw && (off_q < 0 || off_f < 0 || ld_raw < off_q + (int64_t)H * dk || ld_raw < off_f + (int64_t)H * dk)))
+      throw std::invalid_argument("gated_linear_scan: inconsistent sizes");
+    int rc = xgm::gated_linear_scan(P<const float>(q), P<const float>(f), P<const float>(k), P<const void>(raw), ld_raw,
+                                    off_q, off_f, P<const float>(f_bias), P<const float>(lower), P<const void>(v), v_f32,
+                                    ld_v, P<float>(state), P<const int32_t>(qsl), P<const int32_t>(sl),
+                                    P<const int32_t>(slots), P<float>(o), ns, H, dk, dv, S(st));
     check(rc, "gated_linear_scan");
   });
   m.def("ssm_scan", [](uintptr_t xbc, bool f32, int64_t ld_x, uintptr_t dt, int64_t ld_dt, uintptr_t dt_bias,

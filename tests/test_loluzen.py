@@ -542,18 +542,28 @@ def test_gated_linear_recurrence_over_portions_and_slots(device, H, dk, dv):
     n = H * dk
     Wcat = torch.cat([Wt["q"], Wt["f"], Wt["v"]])
     state = torch.randn(3, H, dk, dv).to(device)      # stale contents: a new sequence must not see them
+    state2 = state.clone()
+    fb, low = Wt["f.b"].float().to(device), Wt["lower"].float().to(device)
 
     def fn(x, sm):
         proj = (x.to(F64).cpu() @ Wcat.T).float().to(device)
-        q, f = sq.lower_bound_gates(proj, 0, n, n, Wt["f.b"].float().to(device), Wt["lower"].float().to(device))
+        q, f = sq.lower_bound_gates(proj, 0, n, n, fb, low)
         o = sq.gated_linear_scan(q, f, None, proj[:, 2 * n:], state, H, dk, dv, sm)
         return sq.gated_group_norm(o, None, Wt["norm"].float().to(device), eps, H, torch.float32)
-    got = in_portions(device, hs, [[3, 1, 1, 2, 20, 2], [2, 2, 7]], [1, 2], fn)
-    for h, gt, slot in zip(hs, got, (1, 2)):
-        states = []
-        ref = orc.gated_linear_recurrence(dict(Wt, o=torch.eye(H * dv, dtype=F64)), "", m, h, eps, states)
-        assert rel_err(gt, ref) < 2e-4
-        assert float((state[slot].cpu().to(F64) - torch.stack(states)).abs().max()) < 1e-4
+
+    def fused(x, sm):   # gates formed inside the scan, from columns of a wider row
+        proj = torch.zeros(x.shape[0], Wcat.shape[0] + 5, device=device)
+        proj[:, 5:] = (x.to(F64).cpu() @ Wcat.T).float().to(device)
+        o = sq.lower_bound_recurrence(proj, 5, 5 + n, 5 + 2 * n, fb, low, state2, H, dk, dv, sm)
+        return sq.gated_group_norm(o, None, Wt["norm"].float().to(device), eps, H, torch.float32)
+    cuts = [[3, 1, 1, 2, 20, 2], [2, 2, 7]]
+    for run, st in ((fn, state), (fused, state2)):
+        got = in_portions(device, hs, cuts, [1, 2], run)
+        for h, gt, slot in zip(hs, got, (1, 2)):
+            states = []
+            ref = orc.gated_linear_recurrence(dict(Wt, o=torch.eye(H * dv, dtype=F64)), "", m, h, eps, states)
+            assert rel_err(gt, ref) < 2e-4
+            assert float((st[slot].cpu().to(F64) - torch.stack(states)).abs().max()) < 1e-4
     # a general write strength k (not 1 - f) goes the same way
     T = 13
     q, f, k = torch.rand(T, n, generator=g), torch.rand(T, n, generator=g), torch.randn(T, n, generator=g)

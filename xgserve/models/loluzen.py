@@ -124,8 +124,8 @@ class LowerBoundRecurrence(nn.Module):
 
     def forward(self, proj, sm: sq.SeqMeta, lc: LayerCache):
         n = self.n
-        q, fg = sq.lower_bound_gates(proj, 0, n, n, None, self.lower)   # the gate's bias is in the projection
-        o = sq.gated_linear_scan(q, fg, None, proj[:, 2 * n:], lc.gla, self.H, self.dk, self.dv, sm)
+        # the gate's bias is in the projection
+        o = sq.lower_bound_recurrence(proj, 0, n, 2 * n, None, self.lower, lc.gla, self.H, self.dk, self.dv, sm)
         return F.linear(sq.gated_group_norm(o, None, self.norm, self.eps, self.H, proj.dtype), self.o)
 
 

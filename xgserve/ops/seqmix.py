@@ -434,6 +434,8 @@ def residual_norm(x: torch.Tensor, y1: Optional[torch.Tensor], a1: Optional[torc
 MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
 # XGS_TUNE attn_mfma=0: the general (any size, fp32-capable) kernel for bf16 too (A/B and tests)
 ATTN_MFMA = tune.get_bool("attn_mfma", True)
+# XGS_TUNE attn_waves=4|8|16: waves per workgroup of the matrix-core kernel on prompt portions (0: by portion length)
+ATTN_WAVES = tune.get_int("attn_waves", 0)
 ATTN_MAX_SPLITS = 8      # key shares per single-token row, at most
 ATTN_SPLIT_WGS = 2048    # ... while the launch stays under about this many workgroups
 
@@ -517,7 +519,7 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
                                            _i32(sm.slots).data_ptr(), _p(temp), _p(sink), out.data_ptr(), T, sm.num_seqs,
                                            sm.max_q, H, G, dk, dv, int(mask), int(size), float(scale), nsplit,
                                            _p(part_o), _p(part_ml), _p(gate), gate.stride(0) if gate is not None else 0,
-                                           _p(r1), _p(r2), int(values), stream_ptr())
+                                           _p(r1), _p(r2), int(values), ATTN_WAVES, stream_ptr())
             return out
         mixers().masked_attention(q.data_ptr(), is_f32(q), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(),
                                   bt.shape[1], block_size, _i32(sm.positions).data_ptr(), _i32(sm.token_seq).data_ptr(),
@@ -846,8 +848,8 @@ def gated_linear_scan(q: torch.Tensor, f: torch.Tensor, k: Optional[torch.Tensor
         assert q.dtype == f.dtype == torch.float32 and q.is_contiguous() and f.is_contiguous() and v.stride(1) == 1
         assert k is None or (k.dtype == torch.float32 and k.is_contiguous())
         assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dk, dv)
-        mixers().gated_linear_scan(q.data_ptr(), f.data_ptr(), _p(k), v.data_ptr(), is_f32(v), v.stride(0),
-                                   state.data_ptr(), _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
+        mixers().gated_linear_scan(q.data_ptr(), f.data_ptr(), _p(k), 0, 0, 0, 0, 0, 0, v.data_ptr(), is_f32(v),
+                                   v.stride(0), state.data_ptr(), _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
                                    _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, dk, dv, stream_ptr())
         return o
     qh, fh = q.view(T, H, dk), f.view(T, H, dk)
@@ -863,6 +865,25 @@ def gated_linear_scan(q: torch.Tensor, f: torch.Tensor, k: Optional[torch.Tensor
             S = fh[t][:, :, None] * S + kh[t][:, :, None] * vh[t][:, None, :]
             o[t] = torch.einsum("hkd,hk->hd", S, qh[t]).reshape(H * dv)
         state[slots[s]] = S
+    return o
+
+
+def lower_bound_recurrence(proj: torch.Tensor, off_q: int, off_f: int, off_v: int, f_bias: Optional[torch.Tensor],
+                           lower: torch.Tensor, state: torch.Tensor, H: int, dk: int, dv: int, sm: SeqMeta) -> torch.Tensor:
+    """lower_bound_gates + gated_linear_scan with k = 1 - f on the columns [q | f | v] of one fused projection row:
+    on the GPU the gates are formed while the scan stages its inputs. Returns o fp32 [T, H dv]."""
+    n = H * dk
+    v = proj[:, off_v:off_v + H * dv]
+    if not native_device(proj):
+        q, f = lower_bound_gates(proj, off_q, off_f, n, f_bias, lower)
+        return gated_linear_scan(q, f, None, v, state, H, dk, dv, sm)
+    assert proj.stride(1) == 1 and lower.dtype == torch.float32 and lower.numel() == n
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dk, dv)
+    o = torch.empty(proj.shape[0], H * dv, dtype=torch.float32, device=proj.device)
+    mixers().gated_linear_scan(0, 0, 0, proj.data_ptr(), proj.stride(0), off_q, off_f, _p(f_bias), lower.data_ptr(),
+                               v.data_ptr(), is_f32(proj), proj.stride(0), state.data_ptr(), _i32(sm.qsl).data_ptr(),
+                               _i32(sm.seq_lens).data_ptr(), _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, dk,
+                               dv, stream_ptr())
     return o
 
 
