@@ -9,8 +9,8 @@
 //                      q / f / k are fp32 tensors, or (raw form) q and f are taken straight from the fused
 //                      projection row and pass silu / the lower-bounded sigmoid while they are staged
 //
-// One workgroup = (sequence, head, 64 state columns), NW waves: lane p owns column p, wave w owns rows
-// [w * NI, (w + 1) * NI) of it in registers. f / k / q / v of TT tokens at a time are staged in LDS (two buffers:
+// One workgroup = (sequence, head, 64 or 32 state columns), NW waves: a lane owns one column and NI rows of it in
+// registers (64 columns: wave w owns rows [w * NI, (w + 1) * NI); 32 columns: each half of a wave its own NI rows). f / k / q / v of TT tokens at a time are staged in LDS (two buffers:
 // the next tile's global loads are issued before the current tile's steps and stored after them). Per token
 // a wave does 2 FMAs per owned state element; the waves' partial sums of o meet in LDS once per tile, in
 // wave order.
@@ -32,38 +32,42 @@ __global__ void lower_bound_gates_kernel(const T* __restrict__ proj, int64_t ld,
   f[i] = l + (1.f - l) * sigmoidf(ldf(row + off_f + c) + (f_bias ? f_bias[c] : 0.f));
 }
 
-constexpr int kGlaCols = 64;   // state columns per workgroup
+// State columns per workgroup: COLS = 64 (lane = column) or 32 (lanes 0-31 and 32-63 hold the same 32 columns for
+// different rows, their partial sums meet by one cross-lane add): the narrow form keeps all lanes busy for value sizes
+// up to 32.
 
 // RAW: q and f are read as columns [off_q, off_q + H dk) / [off_f, ..) of the activation rows `raw` and go
 // through silu / the lower-bounded sigmoid while they are staged (no pass of their own, half the bytes), and the
 // write strength is 1 - f. Otherwise q, f (and k, or 1 - f when k == nullptr) are fp32 tensors [T, H dk].
-template <typename T, int NI, int TT, int NW, bool RAW>
+template <typename T, int NI, int TT, int NW, bool RAW, int COLS>
 __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
     const float* __restrict__ q, const float* __restrict__ f, const float* __restrict__ k, const T* __restrict__ raw,
     int64_t ld_raw, int off_q, int off_f, const float* __restrict__ f_bias, const float* __restrict__ lower,
     const T* __restrict__ v, int64_t ld_v, float* __restrict__ state, const int32_t* __restrict__ qsl,
     const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, float* __restrict__ o, int H, int dk,
     int dv) {
-  constexpr int NB = NW * NI;                // padded state rows
+  constexpr int HALVES = 64 / COLS;          // row groups per wave
+  constexpr int NB = NW * HALVES * NI;       // padded state rows
   constexpr int NTH = 64 * NW;
   constexpr int NQ = RAW ? 2 : 3;            // staged row blocks: [f | q | (k)]
-  constexpr int ROW = NQ * NB + kGlaCols;    // staged floats per token: [f | q | (k) | v]
+  constexpr int ROW = NQ * NB + COLS;        // staged floats per token: [f | q | (k) | v]
   constexpr int PER = (TT * ROW + NTH - 1) / NTH;
   __shared__ __attribute__((aligned(16))) float stage[2][TT][ROW];
-  __shared__ float opart[TT][NW][kGlaCols];
+  __shared__ float opart[TT][NW][COLS];
   const int s = blockIdx.x, h = blockIdx.y;
   const int q0 = qsl[s], qn = qsl[s + 1] - q0, slot = slots[s];
   if (slot < 0 || qn <= 0) return;
   const int ctx = seq_lens[s] - qn;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int p0 = blockIdx.z * kGlaCols, p = p0 + lane;
+  const int col = lane % COLS, rg = wave * HALVES + lane / COLS;   // column within the block, row group
+  const int p0 = blockIdx.z * COLS, p = p0 + col;
   const bool pok = p < dv;
   const int nqk = H * dk, nv = H * dv;
   float* Sg = state + (((int64_t)slot * H + h) * dk) * dv;
   float S[NI];
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
-    const int n = wave * NI + i;
+    const int n = rg * NI + i;
     S[i] = (ctx > 0 && pok && n < dk) ? Sg[(int64_t)n * dv + p] : 0.f;
   }
   float pre[PER];
@@ -126,10 +130,10 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
     const bool more = t0 + TT < qn;
     if (more) fetch(t0 + TT);
     auto step = [&](int tt) {
-      const float* fr = &stage[buf][tt][wave * NI];
-      const float* qr = &stage[buf][tt][NB + wave * NI];
-      const float* kr = &stage[buf][tt][(NQ - 1) * NB + wave * NI];   // RAW: unused
-      const float vv = stage[buf][tt][NQ * NB + lane];
+      const float* fr = &stage[buf][tt][rg * NI];
+      const float* qr = &stage[buf][tt][NB + rg * NI];
+      const float* kr = &stage[buf][tt][(NQ - 1) * NB + rg * NI];   // RAW: unused
+      const float vv = stage[buf][tt][NQ * NB + col];
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
@@ -137,7 +141,8 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
         S[i] = RAW ? fmaf(fr[i], S[i] - vv, vv) : fmaf(fr[i], S[i], kr[i] * vv);
         acc = fmaf(S[i], qr[i], acc);
       }
-      opart[tt][wave][lane] = acc;
+      if (HALVES == 2) acc += __shfl_xor(acc, 32, 64);
+      if (lane < COLS) opart[tt][wave][col] = acc;
     };
     if (nt == TT) {  // whole tile: a fixed trip count lets the LDS reads of several steps be in flight together
 #pragma unroll 4
@@ -146,8 +151,8 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
       for (int tt = 0; tt < nt; ++tt) step(tt);
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < nt * kGlaCols; e += NTH) {
-      const int tt = e / kGlaCols, c = e % kGlaCols;
+    for (int e = threadIdx.x; e < nt * COLS; e += NTH) {
+      const int tt = e / COLS, c = e % COLS;
       if (p0 + c < dv) {
         float val = 0.f;
 #pragma unroll
@@ -161,7 +166,7 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
   if (pok) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int n = wave * NI + i;
+      const int n = rg * NI + i;
       if (n < dk) Sg[(int64_t)n * dv + p] = S[i];
     }
   }
@@ -179,14 +184,25 @@ void lower_bound_gates(const void* proj, bool f32, int64_t ld, int off_q, int of
 int gated_linear_scan(const float* q, const float* f, const float* k, const void* raw, int64_t ld_raw, int off_q, int off_f,
                       const float* f_bias, const float* lower, const void* v, bool v_f32, int64_t ld_v, float* state,
                       const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, float* o, int ns, int H, int dk,
-                      int dv, hipStream_t st) {
+                      int dv, int cols_hint, hipStream_t st) {
   if (ns <= 0) return 0;
   if (H <= 0 || dk < 1 || dk > 256 || dv < 1 || (raw ? !lower : (!q || !f))) return -1;
-  dim3 grid(ns, H, (dv + kGlaCols - 1) / kGlaCols);
-#define XGM_GL2(NI, TT, NW, RAW)                                                                                       \
-  XGM_DISPATCH_T(v_f32, gated_linear_scan_kernel<T, NI, TT, NW, RAW><<<grid, 64 * NW, 0, st>>>(                         \
+  // 32-column workgroups for small value sizes (no idle lanes), or on request. Doubling the workgroups of a step that
+  // leaves compute units idle measured no faster: the scan is bound by the latency of a token step, not by lanes.
+  const bool narrow = cols_hint == 32 || (cols_hint != 64 && dv <= 32);
+  const int cols = narrow ? 32 : 64;
+  dim3 grid(ns, H, (dv + cols - 1) / cols);
+#define XGM_GL3(NI, TT, NW, RAW, COLS)                                                                                 \
+  XGM_DISPATCH_T(v_f32, gated_linear_scan_kernel<T, NI, TT, NW, RAW, COLS><<<grid, 64 * NW, 0, st>>>(                   \
                             q, f, k, (const T*)raw, ld_raw, off_q, off_f, f_bias, lower, (const T*)v, ld_v, state, qsl, \
                             seq_lens, slots, o, H, dk, dv);)
+  // NI rows per lane: the narrow form covers twice the rows per wave, so it takes half of them per lane
+#define XGM_GL2(NI, TT, NW, RAW)          \
+  if (narrow) {                           \
+    XGM_GL3((NI / 2), TT, NW, RAW, 32)    \
+  } else {                                \
+    XGM_GL3(NI, TT, NW, RAW, 64)          \
+  }
   // tokens per staged tile: the raw form stages two row blocks instead of three and takes longer tiles
 #define XGM_GL(NI, TT, TTR, NW)           \
   if (raw) {                              \
@@ -202,6 +218,7 @@ int gated_linear_scan(const float* q, const float* f, const float* k, const void
   XGM_GL(32, 4, 4, 8)
 #undef XGM_GL
 #undef XGM_GL2
+#undef XGM_GL3
 }
 
 }  // namespace xgm

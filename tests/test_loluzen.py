@@ -531,7 +531,9 @@ def test_one_standing_out_key_far_back_and_at_page_borders(device, dtype, key, s
 
 @pytest.mark.parametrize("device", OP_CASES)
 @pytest.mark.parametrize("H,dk,dv", [(3, 20, 12), (2, 16, 16), (1, 6, 70), (2, 64, 80), (1, 130, 24)])
-def test_gated_linear_recurrence_over_portions_and_slots(device, H, dk, dv):
+@pytest.mark.parametrize("cols", [32, 64])
+def test_gated_linear_recurrence_over_portions_and_slots(device, H, dk, dv, cols, monkeypatch):
+    monkeypatch.setattr(sq, "SCAN_COLS", cols)    # both workgroup shapes of the scan kernel
     g = torch.Generator().manual_seed(dk)
     W, eps = 24, 1e-5
     m = {"heads": H, "dim": dk, "vdim": dv}

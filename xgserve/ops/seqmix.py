@@ -819,6 +819,10 @@ def talk_mix(o_all: torch.Tensor, talk: torch.Tensor, H: int, G: int, dv: int,
 
 
 # ---------------------------------------------------------------------------- gated linear recurrence
+# XGS_TUNE scan_cols=32|64: state columns per workgroup of the gated linear scan (0: by the size of the step)
+SCAN_COLS = tune.get_int("scan_cols", 0)
+
+
 def lower_bound_gates(proj: torch.Tensor, off_q: int, off_f: int, n: int, f_bias: Optional[torch.Tensor],
                       lower: torch.Tensor):
     """From a fused projection row: q = silu(proj[off_q : off_q + n]) and the forget gate
@@ -850,7 +854,7 @@ def gated_linear_scan(q: torch.Tensor, f: torch.Tensor, k: Optional[torch.Tensor
         assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dk, dv)
         mixers().gated_linear_scan(q.data_ptr(), f.data_ptr(), _p(k), 0, 0, 0, 0, 0, 0, v.data_ptr(), is_f32(v),
                                    v.stride(0), state.data_ptr(), _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
-                                   _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, dk, dv, stream_ptr())
+                                   _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, dk, dv, SCAN_COLS, stream_ptr())
         return o
     qh, fh = q.view(T, H, dk), f.view(T, H, dk)
     kh = (1.0 - fh) if k is None else k.view(T, H, dk)
@@ -883,7 +887,7 @@ def lower_bound_recurrence(proj: torch.Tensor, off_q: int, off_f: int, off_v: in
     mixers().gated_linear_scan(0, 0, 0, proj.data_ptr(), proj.stride(0), off_q, off_f, _p(f_bias), lower.data_ptr(),
                                v.data_ptr(), is_f32(proj), proj.stride(0), state.data_ptr(), _i32(sm.qsl).data_ptr(),
                                _i32(sm.seq_lens).data_ptr(), _i32(sm.slots).data_ptr(), o.data_ptr(), sm.num_seqs, H, dk,
-                               dv, stream_ptr())
+                               dv, SCAN_COLS, stream_ptr())
     return o
 
 
