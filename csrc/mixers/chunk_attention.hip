@@ -520,6 +520,104 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(
     for (int c = threadIdx.x; c < nv; c += blockDim.x) stf(vcache + (int64_t)slot * nv + c, ldf(row + nq + nk + c));
 }
 
+// ------------------------------------------------------------------ short convolution + per-head norm + rotation
+// The same as head_norm_rope_cache on the outputs of a causal depthwise convolution over time of the projected row
+// [q | k | v] (taps <= 8, weights conv_w[channel][tap], no bias), formed here: channel c of the token at local index i
+// of its sequence's rows reads rows i - taps + 1 .. i of this step, or, before the step's first row, the sequence's
+// carried inputs state[slot][taps - 1 + index][c] (zero before the sequence's start). A lane owns the entries
+// d = lane + 64 n (n < NR) of a head, a wave one head, further workgroups the value channels; rotation partners are
+// neighbouring lanes. Steps of single tokens shift the
+// carried inputs here (each thread reads and writes only its own channels); longer steps leave that to a second launch.
+constexpr int kConvMaxTaps = 8;
+
+template <typename TI, typename TO, int NR>
+__global__ __launch_bounds__(256) void conv_head_norm_rope_cache_kernel(
+    const TI* __restrict__ proj, int64_t ld, const float* __restrict__ conv_w, int taps, float* __restrict__ state,
+    const int32_t* __restrict__ qsl, const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots,
+    const int32_t* __restrict__ token_seq, int H, int G, int dk, int dv, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, const float* __restrict__ rot, int rot_rows, int rot_dims,
+    const int32_t* __restrict__ slot_mapping, TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
+    int single) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int nq = H * dk, nk = G * dk, nv = G * dv, C = nq + nk + nv;
+  // blockIdx.y < nhb: one head per wave (H query heads, then G key heads); beyond: 256 value channels per workgroup
+  const int nhb = (H + G + nw - 1) / nw;
+  const int s = token_seq[t];
+  const int slot = s >= 0 ? slots[s] : -1;
+  if (slot < 0) {  // padding row: a defined q row, nothing cached, no state touched
+    const int hd = blockIdx.y * nw + wave;
+    if ((int)blockIdx.y < nhb && hd < H)
+      for (int d = lane; d < dk; d += 64) stf(q_out + (int64_t)t * nq + hd * dk + d, 0.f);
+    return;
+  }
+  const int q0 = qsl[s], qn = qsl[s + 1] - q0;
+  const int ctx = seq_lens[s] - qn, li = t - q0, nh = taps - 1;
+  const int crow = slot_mapping[t];
+  const float* st = state + (int64_t)slot * nh * C;
+  // the convolution of channel c at this token; a single-token step also shifts the channel's carried inputs
+  auto conv = [&](int c) -> float {
+    float u[kConvMaxTaps];
+#pragma unroll
+    for (int j = 0; j < kConvMaxTaps; ++j) {
+      u[j] = 0.f;
+      if (j < taps) {
+        const int idx = li - nh + j;   // local index of the input under tap j
+        if (idx >= 0) u[j] = ldf(proj + (int64_t)(q0 + idx) * ld + c);
+        else if (ctx + idx >= 0) u[j] = st[(int64_t)(nh + idx) * C + c];
+      }
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < kConvMaxTaps; ++j)
+      if (j < taps) acc += conv_w[(int64_t)c * taps + j] * u[j];
+    if (single) {   // carried inputs after this token: u[1 .. taps - 1] (already zero before the sequence's start)
+      float* sw = state + (int64_t)slot * nh * C + c;
+#pragma unroll
+      for (int j = 1; j < kConvMaxTaps; ++j)
+        if (j < taps) sw[(int64_t)(j - 1) * C] = u[j];
+    }
+    return acc;
+  };
+  const float* cs = nullptr;
+  if (rot && rot_dims > 0) cs = rot + (int64_t)min(max(ctx + li, 0), rot_rows - 1) * rot_dims;  // [rot_dims / 2][2]
+  if ((int)blockIdx.y >= nhb) {
+    const int c = ((int)blockIdx.y - nhb) * blockDim.x + threadIdx.x;
+    if (c < nv && (crow >= 0 || single)) {
+      const float v = conv(nq + nk + c);
+      if (crow >= 0) stf(vcache + (int64_t)crow * nv + c, v);
+    }
+    return;
+  }
+  for (int hd = blockIdx.y * nw + wave; hd < H + G; hd += H + G) {   // one pass
+    const bool is_q = hd < H;
+    if (!is_q && crow < 0 && !single) continue;
+    const int c0 = is_q ? hd * dk : nq + (hd - H) * dk;
+    const float* w = is_q ? wq : wk;
+    float a[NR], ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < NR; ++n) {
+      const int d = lane + 64 * n;
+      a[n] = d < dk ? conv(c0 + d) : 0.f;
+      ss += a[n] * a[n];
+    }
+    if (!is_q && crow < 0) continue;
+    const float r = w ? 1.f / sqrtf(wave_sum(ss) / (float)dk + eps) : 1.f;
+    TO* dst = is_q ? q_out + (int64_t)t * nq + hd * dk : kcache + (int64_t)crow * nk + (hd - H) * dk;
+#pragma unroll
+    for (int n = 0; n < NR; ++n) {
+      const int d = lane + 64 * n;
+      float v = d < dk ? a[n] * r * (w ? w[d] : 1.f) : 0.f;
+      const float b = __shfl_xor(v, 1, 64);   // the other entry of the pair (2i, 2i + 1)
+      if (cs && d < rot_dims) {
+        const float c = cs[d & ~1], sn = cs[(d & ~1) + 1];
+        v = (d & 1) ? v * c + b * sn : v * c - b * sn;   // (u, v) -> (u c - v s, v c + u s)
+      }
+      if (d < dk) stf(dst + d, v);
+    }
+  }
+}
+
 // ================================================================== host launchers
 void qk_norm_cache(const void* proj, bool f32, int64_t ld, int nq, int nk, int nv, const float* wq, const float* wk,
                    float eps, const int32_t* slot_mapping, void* q_out, void* kcache, void* vcache, int T_,
@@ -642,6 +740,41 @@ void head_norm_rope_cache(const void* src, bool src_f32, int64_t ld, int H, int 
     if (out_f32) { XGM_HN(bf16, float) } else { XGM_HN(bf16, bf16) }
   }
 #undef XGM_HN
+}
+
+void conv_state_update(const void* x, bool in_f32, int64_t ld_in, float* state, const int32_t* qsl,
+                       const int32_t* seq_lens, const int32_t* slots, int ns, int W, int taps, hipStream_t st);
+
+int conv_head_norm_rope_cache(const void* proj, bool in_f32, int64_t ld, const float* conv_w, int taps, float* state,
+                              const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, const int32_t* token_seq,
+                              int ns, int max_q, int H, int G, int dk, int dv, const float* wq, const float* wk, float eps,
+                              const float* rot, int rot_rows, int rot_dims, const int32_t* slot_mapping, void* q_out,
+                              void* kcache, void* vcache, bool out_f32, int T_, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  if (taps < 1 || taps > kConvMaxTaps || dk > 256 || dk < 1) return -1;
+  const int single = (max_q == 1 && taps > 1) ? 1 : 0;
+  dim3 grid(T_, (H + G + 3) / 4 + (G * dv + 255) / 256);
+#define XGM_CH2(TI, TO, NR)                                                                                          \
+  conv_head_norm_rope_cache_kernel<TI, TO, NR><<<grid, 256, 0, st>>>(                                                \
+      (const TI*)proj, ld, conv_w, taps, state, qsl, seq_lens, slots, token_seq, H, G, dk, dv, wq, wk, eps, rot,     \
+      rot_rows, rot_dims, slot_mapping, (TO*)q_out, (TO*)kcache, (TO*)vcache, single);
+#define XGM_CH(TI, TO)                                                                                               \
+  if (dk <= 64) {                                                                                                    \
+    XGM_CH2(TI, TO, 1)                                                                                               \
+  } else if (dk <= 128) {                                                                                            \
+    XGM_CH2(TI, TO, 2)                                                                                               \
+  } else {                                                                                                           \
+    XGM_CH2(TI, TO, 4)                                                                                               \
+  }
+  if (in_f32) {
+    if (out_f32) { XGM_CH(float, float) } else { XGM_CH(float, bf16) }
+  } else {
+    if (out_f32) { XGM_CH(bf16, float) } else { XGM_CH(bf16, bf16) }
+  }
+#undef XGM_CH
+#undef XGM_CH2
+  if (!single) conv_state_update(proj, in_f32, ld, state, qsl, seq_lens, slots, ns, (H + G) * dk + G * dv, taps, st);
+  return 0;
 }
 
 }  // namespace xgm

@@ -878,6 +878,14 @@ void causal_conv(const void* x, bool in_f32, int64_t ld_in, const float* w, cons
   }
 }
 
+// the carried inputs of a convolution whose outputs another kernel formed: state <- last taps - 1 inputs per sequence
+void conv_state_update(const void* x, bool in_f32, int64_t ld_in, float* state, const int32_t* qsl,
+                       const int32_t* seq_lens, const int32_t* slots, int ns, int W, int taps, hipStream_t st) {
+  if (ns <= 0 || taps <= 1) return;
+  XGM_DISPATCH_T(in_f32, canon_state_kernel<T><<<dim3((W + 255) / 256, ns), 256, 0, st>>>((const T*)x, ld_in, state, qsl,
+                                                                                         seq_lens, slots, W, taps);)
+}
+
 void canon_conv(const float* x, const float* w, float* state, const int32_t* qsl, const int32_t* seq_lens,
                 const int32_t* slots, void* out, bool out_f32, int ns, int max_q, int W, int taps, hipStream_t st) {
   causal_conv(x, true, W, w, nullptr, state, qsl, seq_lens, slots, out, out_f32, ns, max_q, W, taps, true, false, st);

@@ -28,6 +28,9 @@ int masked_attention_mfma(const void*, const void*, const void*, const int32_t*,
 void talk_mix(const void*, bool, const float*, const void*, int64_t, void*, int, int, int, int, hipStream_t);
 void head_norm_rope_cache(const void*, bool, int64_t, int, int, int, int, const float*, const float*, float, const float*,
                           int, int, const int32_t*, const int32_t*, void*, void*, void*, bool, int, hipStream_t);
+int conv_head_norm_rope_cache(const void*, bool, int64_t, const float*, int, float*, const int32_t*, const int32_t*,
+                              const int32_t*, const int32_t*, int, int, int, int, int, int, const float*, const float*,
+                              float, const float*, int, int, const int32_t*, void*, void*, void*, bool, int, hipStream_t);
 int post_norm_residual(float*, const void*, bool, int64_t, const float*, const void*, int64_t, const float*, const float*,
                        const float*, float, const float*, const float*, float, float, void*, bool, int, int, hipStream_t);
 void relu2(const void*, bool, const float*, void*, int64_t, int, hipStream_t);
@@ -157,6 +160,21 @@ PYBIND11_MODULE(_mixers, m) {
                               P<const float>(rot), rot_rows, rot_dims, P<const int32_t>(pos),
                               P<const int32_t>(slot_mapping), P<void>(q_out), P<void>(kc), P<void>(vc), out_f32, T, S(st));
     check(0, "head_norm_rope_cache");
+  });
+  m.def("conv_head_norm_rope_cache", [](uintptr_t proj, bool in_f32, int64_t ld, uintptr_t conv_w, int taps,
+                                        uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t token_seq,
+                                        int ns, int max_q, int H, int G, int dk, int dv, uintptr_t wq, uintptr_t wk,
+                                        float eps, uintptr_t rot, int rot_rows, int rot_dims, uintptr_t slot_mapping,
+                                        uintptr_t q_out, uintptr_t kc, uintptr_t vc, bool out_f32, int T, uintptr_t st) {
+    if (H < 1 || G < 1 || dk < 1 || dv < 1 || ld < (int64_t)(H + G) * dk + (int64_t)G * dv || rot_dims < 0 ||
+        rot_dims > dk || (rot_dims & 1) || (rot && rot_dims > 0 && rot_rows < 1) || (taps > 1 && !state))
+      throw std::invalid_argument("conv_head_norm_rope_cache: inconsistent sizes");
+    int rc = xgm::conv_head_norm_rope_cache(
+        P<const void>(proj), in_f32, ld, P<const float>(conv_w), taps, P<float>(state), P<const int32_t>(qsl),
+        P<const int32_t>(sl), P<const int32_t>(slots), P<const int32_t>(token_seq), ns, max_q, H, G, dk, dv,
+        P<const float>(wq), P<const float>(wk), eps, P<const float>(rot), rot_rows, rot_dims,
+        P<const int32_t>(slot_mapping), P<void>(q_out), P<void>(kc), P<void>(vc), out_f32, T, S(st));
+    check(rc, "conv_head_norm_rope_cache");
   });
   m.def("post_norm_residual", [](uintptr_t x, uintptr_t y, bool y_f32, int64_t ldy, uintptr_t y_bias, uintptr_t y2,
                                  int64_t ldy2, uintptr_t pw1, uintptr_t pw2, uintptr_t post_w, float mult, uintptr_t extra,

@@ -438,13 +438,16 @@ def test_rotation_frequencies_in_all_three_ranges():
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("taps,rot_dims,G", [(1, 0, 1), (3, 8, 2), (4, 24, 4), (8, 10, 2)])
-def test_conv_norm_rotation_attention_over_portions(device, dtype, taps, rot_dims, G):
+@pytest.mark.parametrize("taps,rot_dims,G,dk", [(1, 0, 1, 24), (3, 8, 2, 24), (4, 24, 4, 24), (8, 10, 2, 24), (3, 64, 2, 96),
+                                                 (2, 40, 1, 160)])
+@pytest.mark.parametrize("fused", [True, False], ids=["one-pass", "two-pass"])
+def test_conv_norm_rotation_attention_over_portions(device, dtype, taps, rot_dims, G, dk, fused, monkeypatch):
     """The "attention" mixer alone: carried convolution inputs, per-head norms, rotation by the absolute position,
     pages in a scrambled order, two sequences sharing steps, a slot with another sequence's leftovers."""
+    monkeypatch.setattr(sq, "CONV_PREP_FUSED", fused)   # convolution inside the norm / rotation kernel, or before it
     dt = getattr(torch, dtype)
-    W, H, dk, dv, eps = 40, 4, 24, 12, 1e-5
-    m = {"heads": H, "kv_heads": G, "dim": dk, "vdim": dv, "scale": 0.3, "conv": taps}
+    W, H, dv, eps = 40, 4, 12, 1e-5
+    m = {"heads": H, "kv_heads": G, "dim": dk, "vdim": dv, "scale": 0.3 * (24 / dk) ** 0.5, "conv": taps}
     if rot_dims:
         m["rot"] = {"base": 50.0, "dims": rot_dims, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 24}}
     cfg = {"width": W, "vocab": 8, "layers": [{"type": "attention", "mixer": m, "mlp": None}]}

@@ -68,9 +68,8 @@ class ConvRopeAttention(nn.Module):
 
     def forward(self, h, sm: sq.SeqMeta, lc: LayerCache, block_size: int, rot):
         proj = F.linear(h, self.in_proj)
-        qkv = sq.causal_conv(proj[:, :self.ch], self.conv_w, None, lc.mix_conv, sm, torch.float32)
-        q = sq.head_norm_rope_cache(qkv, self.H, self.G, self.dk, self.dv, self.q_norm, self.k_norm, self.eps, rot,
-                                    self.rot_dims, sm, lc.k, lc.v, h.dtype)
+        q = sq.conv_head_norm_rope_cache(proj, self.conv_w, lc.mix_conv, self.H, self.G, self.dk, self.dv, self.q_norm,
+                                         self.k_norm, self.eps, rot, self.rot_dims, sm, lc.k, lc.v)
         o = sq.masked_attention(q, lc.k, lc.v, self.H, self.G, self.dk, self.dv, sq.MASK_CAUSAL, 0, self.scale, None,
                                 None, block_size, sm, gate=proj[:, self.ch:])
         return F.linear(o, self.o)

@@ -795,6 +795,42 @@ def head_norm_rope_cache(src: torch.Tensor, H: int, G: int, dk: int, dv: int, wq
     return q
 
 
+CONV_PREP_FUSED = tune.get_bool("conv_prep_fused", True)   # XGS_TUNE conv_prep_fused=0: convolution and norm apart
+# steps of more rows run the convolution as a kernel of its own: over a long portion it slides a register window along
+# the tokens (one load per input), where the one-pass kernel loads every tap of every output
+CONV_PREP_FUSED_MAX_ROWS = 1024
+
+
+def conv_head_norm_rope_cache(proj: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, H: int, G: int, dk: int,
+                              dv: int, wq: Optional[torch.Tensor], wk: Optional[torch.Tensor], eps: float,
+                              rot: Optional[torch.Tensor], rot_dims: int, sm: SeqMeta, kcache: torch.Tensor,
+                              vcache: torch.Tensor) -> torch.Tensor:
+    """causal_conv (no bias, no activation) of the columns [q | k | v] of a fused projection row, then
+    head_norm_rope_cache of the result; in one pass on the GPU for steps of single tokens and short portions (the
+    convolution's output never reaches memory).
+    conv_w fp32 [channels, taps]; state fp32 [slots, taps - 1, channels] is updated."""
+    C = (H + G) * dk + G * dv
+    taps = conv_w.shape[1]
+    if not (native_device(proj) and CONV_PREP_FUSED and dk <= 256 and proj.shape[0] <= CONV_PREP_FUSED_MAX_ROWS):
+        qkv = causal_conv(proj[:, :C], conv_w, None, state, sm, torch.float32)
+        return head_norm_rope_cache(qkv, H, G, dk, dv, wq, wk, eps, rot, rot_dims, sm, kcache, vcache, proj.dtype)
+    T = proj.shape[0]
+    q = torch.empty(T, H * dk, dtype=proj.dtype, device=proj.device)
+    assert proj.stride(1) == 1 and conv_w.dtype == torch.float32 and conv_w.is_contiguous() and conv_w.shape[0] == C
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (taps - 1, C)
+    assert kcache.is_contiguous() and vcache.is_contiguous() and kcache.dtype == vcache.dtype == proj.dtype
+    assert kcache.shape[-1] == G * dk and vcache.shape[-1] == G * dv and rot_dims % 2 == 0 and rot_dims <= dk
+    assert rot is None or (rot.dtype == torch.float32 and rot.is_contiguous() and rot.shape[1] * 2 == rot_dims)
+    mixers().conv_head_norm_rope_cache(proj.data_ptr(), is_f32(proj), proj.stride(0), conv_w.data_ptr(), taps,
+                                       state.data_ptr(), _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
+                                       _i32(sm.slots).data_ptr(), _i32(sm.token_seq).data_ptr(), sm.num_seqs, sm.max_q,
+                                       H, G, dk, dv, _p(wq), _p(wk), float(eps), _p(rot),
+                                       rot.shape[0] if rot is not None else 0, rot_dims if rot is not None else 0,
+                                       _i32(sm.slot_mapping).data_ptr(), q.data_ptr(), kcache.data_ptr(),
+                                       vcache.data_ptr(), is_f32(q), T, stream_ptr())
+    return q
+
+
 # ---------------------------------------------------------------------------- mixing the heads' weight maps
 def talk_mix(o_all: torch.Tensor, talk: torch.Tensor, H: int, G: int, dv: int,
              gate: Optional[torch.Tensor] = None) -> torch.Tensor:
