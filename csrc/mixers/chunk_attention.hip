@@ -13,7 +13,7 @@
 //                     the scores only through an optional distance penalty: with r1 / r2 the score of key j
 //                     loses r1[h] * ln(1 + r2[h] * (i - j)). With `gate` head h's output is multiplied by
 //                     sigmoid(gate[t][h]). `vmode` chooses the values a query head weighs: kValuesOwn its own
-//                     key/value head's (output [T][H][dv]), kValuesAll the values of all G heads side by side
+//                     key/value head's (output [T][H][dv]), kValuesAll the concatenated values of all G heads
 //                     (output [T][H][G dv]: what mixing the heads' weight maps after the softmax needs),
 //                     c >= 0 head c's for every query head.
 //   talk_mix          out[t][h] = sigmoid(gate[t][h]) * sum_g talk[h][g] * o_all[t][g][c(h)], c(h) = h / (H / G)

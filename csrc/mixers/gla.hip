@@ -1,5 +1,5 @@
 // Gated linear recurrence with one decay per state row (gated linear attention; with k = 1 - f the
-// forget gate also decides what is written), carried per sequence slot.
+// write strength is the complement of the forget gate), carried per sequence slot.
 //
 //   lower_bound_gates  from a fused projection row: q = silu(z_q);  f = l + (1 - l) * sigmoid(z_f + b)
 //                      (a forget gate bounded below by l, per channel), both fp32

@@ -1,4 +1,4 @@
-"""Loluzen: a decoder with a norm before AND after every sublayer, on the paged / slotted engine.
+"""Loluzen: a decoder whose sublayers are wrapped in two norms (input norm and output norm), on the paged / slotted engine.
 
     x_0 = embed[token] * s                                           (s = cfg.embed_scale)
     x  <- x + m * N(mixer(N(x; norm1)); norm1b)                      (m = cfg.residual_mult)

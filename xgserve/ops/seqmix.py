@@ -490,7 +490,7 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
     otherwise positions do not enter the scores; with `sink` the denominator also holds exp(sink[h]), a term with no
     key and no value; with `gate` ([T, >= H], row-strided) head h's output is multiplied by sigmoid(gate[t, h]).
     `values`: V_OWN: head h weighs the values of its own key/value head, returns [T, H * dv]; V_ALL: the values of
-    all G heads side by side, returns [T, H * G * dv] (what mixing of the heads' weight maps needs);
+    all G heads concatenated, returns [T, H * G * dv] (what mixing of the heads' weight maps needs);
     c >= 0: the values of head c for every query head.
     q [T, H * dk]; caches [rows, G * dk] / [rows, G * dv]."""
     T = q.shape[0]
@@ -711,7 +711,7 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
     return out
 
 
-# ---------------------------------------------------------------------------- norm before and after a sublayer
+# ---------------------------------------------------------------------------- output norm, residual sum, next input norm
 def post_norm_residual(x: torch.Tensor, y: Optional[torch.Tensor], y_bias: Optional[torch.Tensor],
                        post_w: Optional[torch.Tensor], mult: float, extra: Optional[torch.Tensor],
                        next_w: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype] = None,
@@ -880,7 +880,7 @@ def lower_bound_gates(proj: torch.Tensor, off_q: int, off_f: int, n: int, f_bias
 def gated_linear_scan(q: torch.Tensor, f: torch.Tensor, k: Optional[torch.Tensor], v: torch.Tensor, state: torch.Tensor,
                       H: int, dk: int, dv: int, sm: SeqMeta) -> torch.Tensor:
     """Per head a [dk x dv] fp32 state with one decay per row:  S <- diag(f) S + k v^T,  o = S^T q;  k = 1 - f when
-    `k` is None (the forget gate also decides what is written). q, f, k fp32 [T, H dk]; v [T, H dv] (row-strided
+    `k` is None (write strength = complement of the forget gate). q, f, k fp32 [T, H dk]; v [T, H dv] (row-strided
     activation). state fp32 [slots, H, dk, dv] is carried and updated. Returns o fp32 [T, H dv]."""
     T = q.shape[0]
     o = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
