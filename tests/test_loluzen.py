@@ -579,3 +579,73 @@ def test_gated_linear_recurrence_over_portions_and_slots(device, H, dk, dv, cols
     for t in range(T):
         S = f[t].view(H, dk, 1) * S + k[t].view(H, dk, 1).to(F64) * v[t].view(H, 1, dv)
         assert torch.allclose(o[t].to(F64), torch.einsum("hkd,hk->hd", S, q[t].view(H, dk).to(F64)).reshape(-1), atol=1e-4)
+
+
+# ---------------------------------------------------------------------------------- configurations drawn at random
+def _random_config(rng):
+    """Sizes, head counts, taps, rotation settings, layer order and loop drawn independently of each other."""
+    W = rng.choice([64, 96, 160])
+
+    def att():
+        G, rep = rng.choice([1, 2, 3]), rng.choice([1, 2, 5])
+        dk, dv = rng.choice([16, 24, 32, 64, 80]), rng.choice([8, 16, 24, 48])
+        m = {"heads": G * rep, "kv_heads": G, "dim": dk, "vdim": dv, "scale": round(dk ** -0.5 * rng.choice([0.7, 1.3]), 6),
+             "conv": rng.choice([1, 2, 3, 5])}
+        rd = rng.choice([0, 2, dk // 4 * 2, dk])
+        if rd:
+            m["rot"] = {"base": rng.choice([100.0, 10000.0]), "dims": rd}
+            if rng.random() < 0.7:
+                m["rot"]["scaling"] = {"factor": rng.choice([2.0, 8.0]), "low": 1.0, "high": rng.choice([2.0, 4.0]),
+                                       "original": rng.choice([16, 64])}
+        return m
+
+    def par():
+        G, rep = rng.choice([1, 2, 4]), rng.choice([1, 2, 4])
+        dk, dv = rng.choice([16, 32, 48]), rng.choice([16, 32, 48])
+        return {"left": {"heads": G * rep, "kv_heads": G, "dim": dk, "vdim": dv, "scale": round(dk ** -0.5, 6)},
+                "right": {"heads": rng.choice([1, 2, 4]), "dim": rng.choice([8, 16, 64, 96]), "vdim": rng.choice([8, 32, 96])}}
+    n = rng.choice([2, 3, 4])
+    layers = []
+    for _ in range(n):
+        t = rng.choice(["attention", "parallel"])
+        layers.append({"type": t, "mixer": att() if t == "attention" else par(),
+                       "mlp": None if rng.random() < 0.25 else {"kind": "dense", "ff": rng.choice([64, 100])}})
+    a = rng.randrange(0, n)
+    loop = {"start": a, "stop": rng.randrange(a + 1, n + 1), "times": rng.choice([1, 2, 3])} if rng.random() < 0.7 else None
+    return {"architecture": "Loluzen", "width": W, "vocab": rng.choice([97, 300]), "norm": {"eps": rng.choice([1e-5, 1e-6])},
+            "residual_mult": rng.choice([0.3, 1.0]), "embedding": {"scale": round(W ** 0.5, 4)}, "loop": loop, "layers": layers}
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("seed", [3, 14, 15, 92])
+def test_random_configurations_through_mixed_schedules(seed, device, dtype, tmp_path):
+    import random
+    rng = random.Random(seed)
+    cfg = _random_config(rng)
+    Wt = orc.random_weights(cfg, seed)
+    orc.write_checkpoint(str(tmp_path), cfg, Wt)
+    lens = [rng.choice([70, 85]), rng.randrange(2, 20), rng.randrange(20, 45), 1]
+    toks = [tokens_of(cfg, n, seed + i) for i, n in enumerate(lens)]
+    refs = [orc.forward(cfg, Wt, t) for t in toks]
+    eng = engine(str(tmp_path), device, dtype, block_size=16, num_blocks=sum((n + 63) // 64 * 64 for n in lens) // 16,
+                 max_num_seqs=4)
+    at, got = [0] * 4, [[] for _ in lens]
+    while any(at[i] < lens[i] for i in range(4)):
+        entries, who = [], []
+        for i in range(4):
+            if at[i] >= lens[i] or rng.random() < 0.2:
+                continue
+            n = min(lens[i] - at[i], rng.choice([1, 1, 2, 3, 17, 40]))
+            entries.append(("r%d" % i, toks[i][at[i]:at[i] + n], list(range(n))))
+            who.append((i, n))
+            at[i] += n
+        if not entries:
+            continue
+        lg = eng.score_step(entries, ["r%d" % i for i, _ in who if at[i] == lens[i]])
+        o = 0
+        for i, n in who:
+            got[i].append(lg[o:o + n])
+            o += n
+    for i in range(4):
+        assert close(torch.cat(got[i], 0), refs[i], dtype), (i, cfg)
+    assert eng.sched.num_used_blocks() == 0
