@@ -16,6 +16,9 @@
 //                     key/value head's (output [T][H][dv]), kValuesAll the concatenated values of all G heads
 //                     (output [T][H][G dv]: what mixing the heads' weight maps after the softmax needs),
 //                     c >= 0 head c's for every query head.
+//                     `gate_elem`: the gate has one logit per output entry, out[t][h][d] *= sigmoid(gate[t][h dv + d]).
+//                     `wfn` = kWeightsSigmoid: no softmax; the weight of a visible key is sigmoid(score + hbias[h]),
+//                     not normalised over the keys (no sink).
 //   talk_mix          out[t][h] = sigmoid(gate[t][h]) * sum_g talk[h][g] * o_all[t][g][c(h)], c(h) = h / (H / G)
 //   head_norm_rope_cache  per-head RMS norm of q and k (one weight of a head's size for all heads), pairwise
 //                     rotation of each head's first entries by a (cos, sin) table row of the token's position,
@@ -28,6 +31,7 @@ namespace xgm {
 
 constexpr int kMaskCausal = 0, kMaskWindow = 1, kMaskChunk = 2;
 constexpr int kValuesOwn = -1, kValuesAll = -2;
+constexpr int kWeightsSoftmax = 0, kWeightsSigmoid = 1;
 
 __device__ __forceinline__ int first_visible(int mask, int size, int pos) {
   if (mask == kMaskWindow) return max(0, pos - size + 1);
@@ -82,7 +86,8 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
     const int32_t* __restrict__ block_tables, int bt_width, int bs, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ token_seq, const float* __restrict__ temp, const float* __restrict__ sink,
     T* __restrict__ out, int H, int G, int dk, int dv_head, int mask, int size, float scale, int KT,
-    const T* __restrict__ gate, int64_t ld_gate, const float* __restrict__ r1, const float* __restrict__ r2, int vmode) {
+    const T* __restrict__ gate, int64_t ld_gate, const float* __restrict__ r1, const float* __restrict__ r2, int vmode,
+    int gate_elem, int wfn, const float* __restrict__ hbias) {
   extern __shared__ float smem[];
   // dv: value columns per query head; voff: where they start in a cached row of G * dv_head values
   const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
@@ -106,13 +111,14 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
   }
   const int pos = positions[t];
   const int j0 = first_visible(mask, size, pos);
-  float m[kQPW], l[kQPW], acc[kQPW][NR], pen1[kQPW], pen2[kQPW];
+  float m[kQPW], l[kQPW], acc[kQPW][NR], pen1[kQPW], pen2[kQPW], hb[kQPW];
 #pragma unroll
   for (int a = 0; a < kQPW; ++a) {
     const int r = r0 + wave + 4 * a;
     const int h = g * rep + min(r, rep - 1);
     pen1[a] = r1 ? r1[h] : 0.f;
     pen2[a] = r1 ? r2[h] : 0.f;
+    hb[a] = hbias ? hbias[h] : 0.f;
     float* qh = qs + (wave + 4 * a) * dk;
     const float sc = scale * (temp ? temp[h] : 1.f);
     for (int d = lane; d < dk; d += 64) qh[d] = r < rep ? ldf(q + ((int64_t)t * H + h) * dk + d) * sc : 0.f;
@@ -148,14 +154,19 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
       }
       for (int o = 1; o < LPK; o <<= 1) sc += __shfl_xor(sc, o, 64);
       if (r1 && kj < n) sc -= pen1[a] * log1pf(pen2[a] * (float)(pos - (k0 + kj)));
-      if (kj >= n) sc = -INFINITY;
-      const float mn = fmaxf(m[a], wave_max(sc));
-      const float p = kj < n ? expf(sc - mn) : 0.f;
-      const float corr = m[a] == -INFINITY ? 0.f : expf(m[a] - mn);
-      l[a] = l[a] * corr + wave_sum(part == 0 ? p : 0.f);
-      m[a] = mn;
+      float p;
+      if (wfn == kWeightsSigmoid) {   // every visible key weighs sigmoid(score + bias), whatever the others do
+        p = kj < n ? sigmoidf(sc + hb[a]) : 0.f;
+      } else {
+        if (kj >= n) sc = -INFINITY;
+        const float mn = fmaxf(m[a], wave_max(sc));
+        p = kj < n ? expf(sc - mn) : 0.f;
+        const float corr = m[a] == -INFINITY ? 0.f : expf(m[a] - mn);
+        l[a] = l[a] * corr + wave_sum(part == 0 ? p : 0.f);
+        m[a] = mn;
 #pragma unroll
-      for (int i = 0; i < NR; ++i) acc[a][i] *= corr;
+        for (int i = 0; i < NR; ++i) acc[a][i] *= corr;
+      }
       for (int j = 0; j < n; ++j) {
         const float pj = __shfl(p, j * LPK, 64);
 #pragma unroll
@@ -170,12 +181,15 @@ __global__ __launch_bounds__(256) void masked_attention_kernel(
   for (int a = 0; a < kQPW; ++a) {
     const int r = r0 + wave + 4 * a;
     if (r >= rep) continue;
-    float inv = 1.f / l[a];
-    if (gate) inv *= sigmoidf(ldf(gate + (int64_t)t * ld_gate + g * rep + r));
+    float inv = wfn == kWeightsSigmoid ? 1.f : 1.f / l[a];
+    if (gate && !gate_elem) inv *= sigmoidf(ldf(gate + (int64_t)t * ld_gate + g * rep + r));
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       const int d = lane + 64 * i;
-      if (d < dv) stf(out + ((int64_t)t * H + g * rep + r) * dv + d, acc[a][i] * inv);
+      if (d >= dv) continue;
+      float o = acc[a][i] * inv;
+      if (gate && gate_elem) o *= sigmoidf(ldf(gate + (int64_t)t * ld_gate + (int64_t)(g * rep + r) * dv + d));
+      stf(out + ((int64_t)t * H + g * rep + r) * dv + d, o);
     }
   }
 }
@@ -205,7 +219,8 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
     const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, const float* __restrict__ temp,
     const float* __restrict__ sink, bf16* __restrict__ out, int H, int G, int dk, int dv_head, int mask, int size,
     float scale, int RH, int head_slots, float* __restrict__ part_o, float* __restrict__ part_ml, int Ttot,
-    const bf16* __restrict__ gate, int64_t ld_gate, const float* __restrict__ r1, const float* __restrict__ r2, int vmode) {
+    const bf16* __restrict__ gate, int64_t ld_gate, const float* __restrict__ r1, const float* __restrict__ r2, int vmode,
+    int gate_elem, int wfn, const float* __restrict__ hbias) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   // dv: value columns per query head; voff: where they start in a cached row of G * dv_head values
   const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
@@ -274,6 +289,8 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
   // the sink starts the running softmax: weight exp(sink - m) = 1 with no value behind it
   const bool with_sink = sink && (nsplit == 1 || blockIdx.x == 0);  // the sink enters the first share only
   float m = with_sink ? sink[head] * kLog2e : -INFINITY, l = with_sink ? 1.f : 0.f;
+  const bool sig = wfn == kWeightsSigmoid;
+  const float sbias = (sig && hbias) ? hbias[head] * kLog2e : 0.f;   // the per-head score bias, in units of ln 2
 
   // staging: thread -> (row = tid / NW, 16-byte chunks tid % NW, + NW, ..) of the K row and of the V row. The next
   // tile's rows are loaded into registers before the current tile's products and stored after them.
@@ -340,27 +357,35 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
         sacc[n][r] = v;
         mx = fmaxf(mx, v);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = (m_new == -INFINITY || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : exp2_fast(m - m_new);
-    float rs = 0.f;
+    if (sig) {
+      // weight = sigmoid(score + bias) = 1 / (1 + 2^-(s + b)) with s, b in units of ln 2; an unseen key (-inf) weighs 0
 #pragma unroll
-    for (int n = 0; n < 4; ++n)
+      for (int n = 0; n < 4; ++n)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = m_new == -INFINITY ? 0.f : exp2_fast(sacc[n][r] - m_new);
-        sacc[n][r] = p;
-        rs += p;
-      }
-    rs += __shfl_xor(rs, 16, 64);
-    rs += __shfl_xor(rs, 32, 64);
-    l = l * alpha + rs;
-    m = m_new;
+        for (int r = 0; r < 4; ++r) sacc[n][r] = __frcp_rn(1.f + exp2_fast(-(sacc[n][r] + sbias)));
+    } else {
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m, mx);
+      const float alpha = (m_new == -INFINITY || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : exp2_fast(m - m_new);
+      float rs = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < NMT_MAX; ++mt)
+      for (int n = 0; n < 4; ++n)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[mt][r] *= alpha;
+        for (int r = 0; r < 4; ++r) {
+          const float p = m_new == -INFINITY ? 0.f : exp2_fast(sacc[n][r] - m_new);
+          sacc[n][r] = p;
+          rs += p;
+        }
+      rs += __shfl_xor(rs, 16, 64);
+      rs += __shfl_xor(rs, 32, 64);
+      l = l * alpha + rs;
+      m = m_new;
+#pragma unroll
+      for (int mt = 0; mt < NMT_MAX; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[mt][r] *= alpha;
+    }
     // O^T += V^T . P^T over two 32-key halves (keys in the order the score accumulator holds them)
 #pragma unroll
     for (int sc = 0; sc < 2; ++sc) {
@@ -393,15 +418,21 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
       if (mt < nmt)
         *reinterpret_cast<float4*>(part_o + row * dv + mt * 16 + 4 * kg) = make_float4(o[mt][0], o[mt][1], o[mt][2], o[mt][3]);
   } else if (valid) {
-    float inv = l > 0.f ? 1.f / l : 0.f;
-    if (gate) inv *= sigmoidf(bf2f(gate[(int64_t)(q0 + tok) * ld_gate + head]));
+    float inv = sig ? 1.f : (l > 0.f ? 1.f / l : 0.f);
+    if (gate && !gate_elem) inv *= sigmoidf(bf2f(gate[(int64_t)(q0 + tok) * ld_gate + head]));
     bf16* op = out + ((int64_t)(q0 + tok) * H + head) * dv;
+    const bf16* ge = gate_elem ? gate + (int64_t)(q0 + tok) * ld_gate + (int64_t)head * dv : nullptr;
 #pragma unroll
     for (int mt = 0; mt < NMT_MAX; ++mt)
       if (mt < nmt) {
+        float e[4] = {o[mt][0] * inv, o[mt][1] * inv, o[mt][2] * inv, o[mt][3] * inv};
+        if (ge) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) e[r] *= sigmoidf(bf2f(ge[mt * 16 + 4 * kg + r]));
+        }
         uint2 w;
-        w.x = xgk::pack2(o[mt][0] * inv, o[mt][1] * inv);
-        w.y = xgk::pack2(o[mt][2] * inv, o[mt][3] * inv);
+        w.x = xgk::pack2(e[0], e[1]);
+        w.y = xgk::pack2(e[2], e[3]);
         *reinterpret_cast<uint2*>(op + mt * 16 + 4 * kg) = w;
       }
   }
@@ -410,9 +441,20 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
 // merge the key shares of a single-token step: out = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s (m in units of ln 2)
 __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                 const int32_t* __restrict__ slots, bf16* __restrict__ out, int Ttot, int H,
-                                                int dv, int nsplit, const bf16* __restrict__ gate, int64_t ld_gate) {
+                                                int dv, int nsplit, const bf16* __restrict__ gate, int64_t ld_gate,
+                                                int gate_elem, int wfn) {
   const int t = blockIdx.x, h = blockIdx.y;
   if (slots[t] < 0) return;  // single-token steps: row t is sequence t (its output row was zeroed)
+  if (wfn == kWeightsSigmoid) {   // unnormalised weights: the shares simply add up
+    const float gh = (gate && !gate_elem) ? sigmoidf(bf2f(gate[(int64_t)t * ld_gate + h])) : 1.f;
+    for (int d = threadIdx.x; d < dv; d += blockDim.x) {
+      float acc = 0.f;
+      for (int sp = 0; sp < nsplit; ++sp) acc += part_o[(((int64_t)sp * Ttot + t) * H + h) * dv + d];
+      if (gate && gate_elem) acc *= sigmoidf(bf2f(gate[(int64_t)t * ld_gate + (int64_t)h * dv + d]));
+      out[((int64_t)t * H + h) * dv + d] = f2bf(acc * gh);
+    }
+    return;
+  }
   float M = -INFINITY;
   for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, part_ml[2 * (((int64_t)sp * Ttot + t) * H + h)]);
   float L = 0.f;
@@ -422,7 +464,7 @@ __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o
     if (ms != -INFINITY) L += exp2_fast(ms - M) * part_ml[2 * row + 1];
   }
   float inv = L > 0.f ? 1.f / L : 0.f;
-  if (gate) inv *= sigmoidf(bf2f(gate[(int64_t)t * ld_gate + h]));
+  if (gate && !gate_elem) inv *= sigmoidf(bf2f(gate[(int64_t)t * ld_gate + h]));
   for (int d = threadIdx.x; d < dv; d += blockDim.x) {
     float acc = 0.f;
     for (int sp = 0; sp < nsplit; ++sp) {
@@ -430,7 +472,9 @@ __global__ void masked_attention_combine_kernel(const float* __restrict__ part_o
       const float ms = part_ml[2 * row];
       if (ms != -INFINITY) acc += exp2_fast(ms - M) * part_o[row * dv + d];
     }
-    out[((int64_t)t * H + h) * dv + d] = f2bf(acc * inv);
+    acc *= inv;
+    if (gate && gate_elem) acc *= sigmoidf(bf2f(gate[(int64_t)t * ld_gate + (int64_t)h * dv + d]));
+    out[((int64_t)t * H + h) * dv + d] = f2bf(acc);
   }
 }
 
@@ -475,15 +519,20 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(const T* __restrict__ o_a
   }
 }
 
-// ------------------------------------------------------------------ per-head norm + rotation -> q, cache rows
+// ------------------------------------------------------------------ q / k norm + rotation -> q, cache rows
 // One workgroup per token; a wave takes the heads (H query heads, then G key heads) round robin. A lane owns the
 // entries d = lane, lane + 64, ... of a head; the partner of a rotated entry is re-read (it is in the same row).
+// whole: q and k are normed over all their entries at once (weights of size H dk / G dk) instead of head by head.
+// half: the rotation pairs entry i with i + rot_dims / 2 instead of 2i with 2i + 1.
+// v_first / v_mix: the cached values are (1 - lambda) v + lambda v_first, lambda = *v_mix.
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(
     const TI* __restrict__ src, int64_t ld, int H, int G, int dk, int dv, const float* __restrict__ wq,
     const float* __restrict__ wk, float eps, const float* __restrict__ rot, int rot_rows, int rot_dims,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_mapping, TO* __restrict__ q_out,
-    TO* __restrict__ kcache, TO* __restrict__ vcache) {
+    TO* __restrict__ kcache, TO* __restrict__ vcache, int whole, int half, const TI* __restrict__ v_first,
+    int64_t ld_vf, const float* __restrict__ v_mix) {
+  __shared__ float red[4];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const TI* row = src + (int64_t)t * ld;
@@ -491,14 +540,36 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(
   const int nq = H * dk, nk = G * dk, nv = G * dv;
   const float* cs = nullptr;
   if (rot && rot_dims > 0) cs = rot + (int64_t)min(max(positions[t], 0), rot_rows - 1) * rot_dims;  // [rot_dims / 2][2]
+  float rq = 1.f, rk = 1.f;
+  if (whole) {
+    if (wq) {
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < nq; c += blockDim.x) {
+        const float a = ldf(row + c);
+        ss += a * a;
+      }
+      rq = 1.f / sqrtf(block_sum(ss, red) / (float)nq + eps);
+    }
+    if (wk) {
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < nk; c += blockDim.x) {
+        const float a = ldf(row + nq + c);
+        ss += a * a;
+      }
+      rk = 1.f / sqrtf(block_sum(ss, red) / (float)nk + eps);
+    }
+  }
+  const int hr = rot_dims / 2;
   for (int hd = wave; hd < H + G; hd += nw) {
     const bool is_q = hd < H;
     if (!is_q && slot < 0) continue;   // padding row: nothing is cached
-    const TI* v = row + (is_q ? hd * dk : nq + (hd - H) * dk);
+    const int hh = is_q ? hd : hd - H;
+    const TI* v = row + (is_q ? hd * dk : nq + hh * dk);
     const float* w = is_q ? wq : wk;
-    TO* dst = is_q ? q_out + (int64_t)t * nq + hd * dk : kcache + (int64_t)slot * nk + (hd - H) * dk;
-    float r = 1.f;
-    if (w) {
+    const float* wh = (w && whole) ? w + hh * dk : w;   // this head's weights
+    TO* dst = is_q ? q_out + (int64_t)t * nq + hd * dk : kcache + (int64_t)slot * nk + hh * dk;
+    float r = is_q ? rq : rk;
+    if (w && !whole) {
       float ss = 0.f;
       for (int d = lane; d < dk; d += 64) {
         const float a = ldf(v + d);
@@ -507,17 +578,28 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(
       r = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
     }
     for (int d = lane; d < dk; d += 64) {
-      float a = ldf(v + d) * r * (w ? w[d] : 1.f);
+      float a = ldf(v + d) * r * (w ? wh[d] : 1.f);
       if (cs && d < rot_dims) {
-        const float b = ldf(v + (d ^ 1)) * r * (w ? w[d ^ 1] : 1.f);
-        const float c = cs[d & ~1], sn = cs[(d & ~1) + 1];
-        a = (d & 1) ? a * c + b * sn : a * c - b * sn;   // (u, v) -> (u c - v s, v c + u s)
+        const int pd = half ? (d < hr ? d + hr : d - hr) : (d ^ 1);     // the other entry of the pair
+        const bool second = half ? d >= hr : (d & 1);
+        const int pi = half ? (d < hr ? d : d - hr) : (d >> 1);         // the pair's index
+        const float b = ldf(v + pd) * r * (w ? wh[pd] : 1.f);
+        const float c = cs[2 * pi], sn = cs[2 * pi + 1];
+        a = second ? a * c + b * sn : a * c - b * sn;   // (u, v) -> (u c - v s, v c + u s)
       }
       stf(dst + d, a);
     }
   }
-  if (slot >= 0)
-    for (int c = threadIdx.x; c < nv; c += blockDim.x) stf(vcache + (int64_t)slot * nv + c, ldf(row + nq + nk + c));
+  if (slot >= 0) {
+    if (v_first) {
+      const float lam = *v_mix;
+      for (int c = threadIdx.x; c < nv; c += blockDim.x)
+        stf(vcache + (int64_t)slot * nv + c,
+            (1.f - lam) * ldf(row + nq + nk + c) + lam * ldf(v_first + (int64_t)t * ld_vf + c));
+    } else {
+      for (int c = threadIdx.x; c < nv; c += blockDim.x) stf(vcache + (int64_t)slot * nv + c, ldf(row + nq + nk + c));
+    }
+  }
 }
 
 // ------------------------------------------------------------------ short convolution + per-head norm + rotation
@@ -632,7 +714,8 @@ static int launch_masked_attention(const void* q, const void* kcache, const void
                                    int bt_width, int bs, const int32_t* positions, const int32_t* token_seq,
                                    const float* temp, const float* sink, void* out, int T_, int H, int G, int dk,
                                    int dv_head, int mask, int size, float scale, const void* gate, int64_t ld_gate,
-                                   const float* r1, const float* r2, int vmode, hipStream_t st) {
+                                   const float* r1, const float* r2, int vmode, int gate_elem, int wfn,
+                                   const float* hbias, hipStream_t st) {
   const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
   int KT = 64;
   auto bytes = [&](int kt) { return ((size_t)kt * (dk + dv + 2) + (size_t)4 * kQPW * dk) * sizeof(float); };
@@ -643,7 +726,8 @@ static int launch_masked_attention(const void* q, const void* kcache, const void
   masked_attention_kernel<T, NR><<<grid, 256, bytes(KT), st>>>((const T*)q, (const T*)kcache, (const T*)vcache,
                                                                block_tables, bt_width, bs, positions, token_seq, temp,
                                                                sink, (T*)out, H, G, dk, dv_head, mask, size, scale, KT,
-                                                               (const T*)gate, ld_gate, r1, r2, vmode);
+                                                               (const T*)gate, ld_gate, r1, r2, vmode, gate_elem, wfn,
+                                                               hbias);
   return 0;
 }
 
@@ -651,16 +735,18 @@ int masked_attention(const void* q, bool f32, const void* kcache, const void* vc
                      int bt_width, int bs, const int32_t* positions, const int32_t* token_seq, const float* temp,
                      const float* sink, void* out, int T_, int H, int G, int dk, int dv_head, int mask, int size,
                      float scale, const void* gate, int64_t ld_gate, const float* r1, const float* r2, int vmode,
-                     hipStream_t st) {
+                     bool gate_elem, int wfn, const float* hbias, hipStream_t st) {
   if (T_ <= 0) return 0;
   const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
   if (G <= 0 || H % G != 0 || dk <= 0 || dv <= 0 || dv > 512 || mask < 0 || mask > 2 ||
-      (mask != kMaskCausal && size < 1) || vmode < kValuesAll || vmode >= G || (r1 && !r2))
+      (mask != kMaskCausal && size < 1) || vmode < kValuesAll || vmode >= G || (r1 && !r2) ||
+      (gate_elem && vmode != kValuesOwn) || wfn < 0 || wfn > 1 || (wfn == kWeightsSigmoid && sink))
     return -1;
 #define XGM_MA(NR)                                                                                                     \
   XGM_DISPATCH_T(f32, return (launch_masked_attention<T, NR>(q, kcache, vcache, block_tables, bt_width, bs, positions, \
                                                              token_seq, temp, sink, out, T_, H, G, dk, dv_head, mask,  \
-                                                             size, scale, gate, ld_gate, r1, r2, vmode, st));)
+                                                             size, scale, gate, ld_gate, r1, r2, vmode,             \
+                                                             gate_elem ? 1 : 0, wfn, hbias, st));)
   if (dv <= 64) { XGM_MA(1) }
   if (dv <= 128) { XGM_MA(2) }
   if (dv <= 256) { XGM_MA(4) }
@@ -673,12 +759,15 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
                           int bs, const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, const float* temp,
                           const float* sink, void* out, int T_, int ns, int max_q, int H, int G, int dk, int dv_head,
                           int mask, int size, float scale, int nsplit, float* part_o, float* part_ml, const void* gate,
-                          int64_t ld_gate, const float* r1, const float* r2, int vmode, int nw_hint, hipStream_t st) {
+                          int64_t ld_gate, const float* r1, const float* r2, int vmode, int nw_hint, bool gate_elem,
+                          int wfn, const float* hbias, hipStream_t st) {
   if (T_ <= 0 || ns <= 0 || max_q <= 0) return 0;
   const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
   if (G <= 0 || H % G != 0 || dk % 32 != 0 || dv % 16 != 0 || dk > 128 || dv > 256 || mask < 0 || mask > 2 ||
-      (mask != kMaskCausal && size < 1) || vmode < kValuesAll || vmode >= G || (r1 && !r2))
+      (mask != kMaskCausal && size < 1) || vmode < kValuesAll || vmode >= G || (r1 && !r2) ||
+      (gate_elem && vmode != kValuesOwn) || wfn < 0 || wfn > 1 || (wfn == kWeightsSigmoid && sink))
     return -1;
+  const int ge = gate_elem ? 1 : 0;
   const int rep = H / G;
   const int RH = rep >= 4 ? 4 : rep >= 2 ? 2 : 1;
   // a step of single tokens: one workgroup per (sequence, key/value head), its query heads as the slots
@@ -697,7 +786,7 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
   masked_attention_mfma_kernel<NKK, NMT, NW><<<grid, 64 * NW, lds, st>>>(                                             \
       (const bf16*)q, (const bf16*)kcache, (const bf16*)vcache, block_tables, bt_width, bs, qsl, seq_lens, slots, temp, \
       sink, (bf16*)out, H, G, dk, dv_head, mask, size, scale, RH, head_slots, part_o, part_ml, T_, (const bf16*)gate,  \
-      ld_gate, r1, r2, vmode);
+      ld_gate, r1, r2, vmode, ge, wfn, hbias);
 #define XGM_MM(NKK, NMT)                                                                                              \
   if (nw == 16 && NMT <= 8) {                                                                                         \
     XGM_MK(NKK, NMT, (NMT <= 8 ? 16 : 8))                                                                             \
@@ -708,7 +797,7 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
   }                                                                                                                   \
   if (nsplit > 1)                                                                                                     \
     masked_attention_combine_kernel<<<dim3(T_, H), 64, 0, st>>>(part_o, part_ml, slots, (bf16*)out, T_, H, dv, nsplit, \
-                                                                (const bf16*)gate, ld_gate);                          \
+                                                                (const bf16*)gate, ld_gate, ge, wfn);                 \
   return 0;
   if (dk <= 64 && dv <= 64) { XGM_MM(2, 4) }
   if (dk <= 128 && dv <= 128) { XGM_MM(4, 8) }
@@ -728,12 +817,14 @@ void talk_mix(const void* o_all, bool f32, const float* talk, const void* gate, 
 void head_norm_rope_cache(const void* src, bool src_f32, int64_t ld, int H, int G, int dk, int dv, const float* wq,
                           const float* wk, float eps, const float* rot, int rot_rows, int rot_dims,
                           const int32_t* positions, const int32_t* slot_mapping, void* q_out, void* kcache, void* vcache,
-                          bool out_f32, int T_, hipStream_t st) {
+                          bool out_f32, int T_, bool whole, bool half, const void* v_first, int64_t ld_vf,
+                          const float* v_mix, hipStream_t st) {
   if (T_ <= 0) return;
 #define XGM_HN(TI, TO)                                                                                               \
   head_norm_rope_cache_kernel<TI, TO><<<T_, 256, 0, st>>>((const TI*)src, ld, H, G, dk, dv, wq, wk, eps, rot, rot_rows, \
                                                           rot_dims, positions, slot_mapping, (TO*)q_out, (TO*)kcache,  \
-                                                          (TO*)vcache);
+                                                          (TO*)vcache, whole ? 1 : 0, half ? 1 : 0, (const TI*)v_first, \
+                                                          ld_vf, v_mix);
   if (src_f32) {
     if (out_f32) { XGM_HN(float, float) } else { XGM_HN(float, bf16) }
   } else {

@@ -3,6 +3,8 @@
 //
 //   lower_bound_gates  from a fused projection row: q = silu(z_q);  f = l + (1 - l) * sigmoid(z_f + b)
 //                      (a forget gate bounded below by l, per channel), both fp32
+//   decay_gates        q = z_q * q_scale, k = z_k and a decay per key channel f = sigmoid(z + b)^(1 / tau),
+//                      evaluated as exp(-softplus(-(z + b)) / tau), all fp32 (the inputs of gated_linear_scan with k)
 //   gated_linear_scan  per head, state S [dk x dv] fp32 per (slot, head):
 //                        S_t = diag(f_t) S_(t-1) + k_t v_t^T        (k_t = 1 - f_t when k == nullptr)
 //                        o_t = S_t^T q_t
@@ -30,6 +32,21 @@ __global__ void lower_bound_gates_kernel(const T* __restrict__ proj, int64_t ld,
   q[i] = siluf(ldf(row + off_q + c));
   const float l = lower[c];
   f[i] = l + (1.f - l) * sigmoidf(ldf(row + off_f + c) + (f_bias ? f_bias[c] : 0.f));
+}
+
+template <typename T>
+__global__ void decay_gates_kernel(const T* __restrict__ proj, int64_t ld, int off_q, int off_k, int n, float q_scale,
+                                   const T* __restrict__ z, int64_t ld_z, const float* __restrict__ z_bias, float inv_tau,
+                                   float* __restrict__ q, float* __restrict__ f, float* __restrict__ k, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / n;
+  const int c = (int)(i % n);
+  const T* row = proj + t * ld;
+  q[i] = ldf(row + off_q + c) * q_scale;
+  k[i] = ldf(row + off_k + c);
+  const float zz = ldf(z + t * ld_z + c) + (z_bias ? z_bias[c] : 0.f);
+  f[i] = expf(-softplusf(-zz) * inv_tau);   // log sigmoid(z) = -softplus(-z)
 }
 
 // State columns per workgroup: COLS = 64 (lane = column) or 32 (lanes 0-31 and 32-63 hold the same 32 columns for
@@ -179,6 +196,14 @@ void lower_bound_gates(const void* proj, bool f32, int64_t ld, int off_q, int of
   const int64_t total = (int64_t)T_ * n;
   XGM_DISPATCH_T(f32, lower_bound_gates_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(
                           (const T*)proj, ld, off_q, off_f, n, f_bias, lower, q, f, total);)
+}
+
+void decay_gates(const void* proj, bool f32, int64_t ld, int off_q, int off_k, int n, float q_scale, const void* z,
+                 int64_t ld_z, const float* z_bias, float inv_tau, float* q, float* f, float* k, int T_, hipStream_t st) {
+  if (T_ <= 0 || n <= 0) return;
+  const int64_t total = (int64_t)T_ * n;
+  XGM_DISPATCH_T(f32, decay_gates_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(
+                          (const T*)proj, ld, off_q, off_k, n, q_scale, (const T*)z, ld_z, z_bias, inv_tau, q, f, k, total);)
 }
 
 int gated_linear_scan(const float* q, const float* f, const float* k, const void* raw, int64_t ld_raw, int off_q, int off_f,

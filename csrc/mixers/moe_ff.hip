@@ -9,9 +9,14 @@
 //                    others are excluded outright: selection score -inf); the `top` highest eligible selection
 //                    scores win; weight = score * scale (the correction does not enter it, no normalisation)
 //   moe_align        (token, choice) pairs sorted by expert into tiles of `tm` rows (padded with -1)
-//   grouped_gemm     per tile: rows x expert weights; first GEMM with the gated activation fused,
-//                    second GEMM to fp32 rows
-//   moe_combine      out[t] = sum_j weight[t, j] * y[row of pair (t, j)]   (fixed order: bit-stable)
+//   grouped_gemm     per tile: rows x expert weights, in one of three modes:
+//                      kGemmRows    A rows as they lie in the sorted layout -> fp32 rows (the second product)
+//                      kGemmGated   A rows gathered by token; weights [gate | up]; output glu(gate, up)
+//                      kGemmAct     A rows gathered by token; output act(s * (W a)), s = row_scale[pair] (nullptr = 1):
+//                                   a routing weight that multiplies the expert's INPUT is applied to the fp32
+//                                   accumulator of the (linear) first product.  kActRelu2: max(z, 0)^2
+//   moe_combine      out[t] = sum_j weight[t, j] * y[row of pair (t, j)]   (fixed order: bit-stable; weights
+//                    nullptr = 1)
 //
 // Activations / weights are T = float or bf16; router, weights of the sum and the sum itself are fp32.
 #include "mixers_common.h"
@@ -20,7 +25,14 @@
 
 namespace xgm {
 
-constexpr int kGluGeluTanh = 0, kGluClamped = 1;
+constexpr int kGluGeluTanh = 0, kGluClamped = 1, kActRelu2 = 2;
+constexpr int kGemmRows = 0, kGemmGated = 1, kGemmAct = 2;
+
+__device__ __forceinline__ float act1(int kind, float z) {
+  (void)kind;  // kActRelu2
+  const float r = fmaxf(z, 0.f);
+  return r * r;
+}
 
 __device__ __forceinline__ float glu(int kind, float g, float u, float limit, float alpha) {
   if (kind == kGluGeluTanh) {
@@ -154,12 +166,13 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restri
 // columns tc + 16 j. K runs through LDS in chunks of 32. GATED: the weight holds [gate (F rows) | up (F rows)]
 // and the output column f is glu(gate_f, up_f); A rows are gathered through rows[] / top. `tm` = rows per
 // expert tile of the layout (a multiple of 16).
-template <typename T, bool GATED>
+template <typename T, int MODE>
 __global__ __launch_bounds__(256) void grouped_gemm_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ Wt,
                                                            const int32_t* __restrict__ rows,
                                                            const int32_t* __restrict__ tile_expert, int tm, int top,
                                                            int Nout, int K, void* __restrict__ out, int kind, float limit,
-                                                           float alpha) {
+                                                           float alpha, const float* __restrict__ row_scale) {
+  constexpr bool GATED = MODE == kGemmGated, FIRST = MODE != kGemmRows;
   __shared__ float As[16][33];
   __shared__ float Ws[64][33];
   __shared__ float Us[GATED ? 64 : 1][33];
@@ -179,7 +192,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const T* __restrict__
       const int rr = i >> 5, kk = i & 31;
       const int p2 = rows[rbase + rr];
       float v = 0.f;
-      if (p2 >= 0 && k0 + kk < K) v = ldf(A + (int64_t)(GATED ? p2 / top : rbase + rr) * lda + k0 + kk);
+      if (p2 >= 0 && k0 + kk < K) v = ldf(A + (int64_t)(FIRST ? p2 / top : rbase + rr) * lda + k0 + kk);
       As[rr][kk] = v;
     }
     for (int i = threadIdx.x; i < 64 * 32; i += 256) {
@@ -205,6 +218,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const T* __restrict__
     const int n = n0 + tc + 16 * j;
     if (n >= Nout) continue;
     if (GATED) stf((T*)out + (int64_t)r * Nout + n, glu(kind, acc[j], accu[j], limit, alpha));
+    else if (FIRST) stf((T*)out + (int64_t)r * Nout + n, act1(kind, acc[j] * (row_scale ? row_scale[pr] : 1.f)));
     else ((float*)out)[(int64_t)r * Nout + n] = acc[j];
   }
 }
@@ -221,13 +235,15 @@ using xgk::f32x4_t;
 using xgk::ld16;
 using xgk::mfma16x16x32;
 
-template <bool GATED, int MT, int NT, bool SPLITK, bool K64>
+template <int MODE, int MT, int NT, bool SPLITK, bool K64>
 __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __restrict__ A, int64_t lda,
                                                                 const bf16* __restrict__ Wt,
                                                                 const int32_t* __restrict__ rows,
                                                                 const int32_t* __restrict__ tile_expert, int top,
                                                                 int Nout, int K, void* __restrict__ out, int kind,
-                                                                float limit, float alpha) {
+                                                                float limit, float alpha,
+                                                                const float* __restrict__ row_scale) {
+  constexpr bool GATED = MODE == kGemmGated, FIRST = MODE != kGemmRows;
   constexpr int NG = GATED ? NT : 1;
   __shared__ float red[SPLITK ? 3 : 1][SPLITK ? (NT + NG) : 1][64][4];
   const int tile = blockIdx.x;          // layout tile of 16 MT rows
@@ -246,7 +262,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
   for (int i = 0; i < MT; ++i) {
     const int pa = rows[rbase + 16 * i + l16];
     aok[i] = pa >= 0;
-    arow[i] = A + (int64_t)(GATED ? max(pa, 0) / top : rbase + 16 * i + l16) * lda + kg * (K64 ? 16 : 8);
+    arow[i] = A + (int64_t)(FIRST ? max(pa, 0) / top : rbase + 16 * i + l16) * lda + kg * (K64 ? 16 : 8);
   }
   f32x4_t acc[MT][NT], accu[MT][NG];
 #pragma unroll
@@ -327,8 +343,10 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int rr = rbase + 16 * i + kg * 4 + r;
-        if (rows[rr] < 0) continue;
+        const int pr = rows[rr];
+        if (pr < 0) continue;
         if (GATED) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(glu(kind, acc[i][j][r], accu[i][GATED ? j : 0][r], limit, alpha));
+        else if (FIRST) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(act1(kind, acc[i][j][r] * (row_scale ? row_scale[pr] : 1.f)));
         else ((float*)out)[(int64_t)rr * Nout + n] = acc[i][j][r];
       }
     }
@@ -337,13 +355,15 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
 // ---- prompt-sized steps (layout tiles of 64 or 128 rows): a workgroup owns 16 MT rows x 4 x 16 NT columns. The A rows
 // (gathered token rows, shared by the four waves) go through LDS, 32 k at a time in two buffers, one barrier
 // per step; every wave streams its own B columns from global memory into registers.
-template <bool GATED, int MT, int NT>
+template <int MODE, int MT, int NT>
 __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* __restrict__ A, int64_t lda,
                                                                     const bf16* __restrict__ Wt,
                                                                     const int32_t* __restrict__ rows,
                                                                     const int32_t* __restrict__ tile_expert, int tm,
                                                                     int top, int Nout, int K, void* __restrict__ out,
-                                                                    int kind, float limit, float alpha) {
+                                                                    int kind, float limit, float alpha,
+                                                                    const float* __restrict__ row_scale) {
+  constexpr bool GATED = MODE == kGemmGated, FIRST = MODE != kGemmRows;
   constexpr int LDA = 40, NG = GATED ? NT : 1, RPT = MT / 4;  // RPT: staged rows per thread
   __shared__ __attribute__((aligned(16))) uint16_t As[2][16 * MT * LDA];
   const int tile = blockIdx.x;  // 16 MT rows of a layout tile of tm rows
@@ -362,7 +382,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* 
 #pragma unroll
   for (int r = 0; r < RPT; ++r) {
     pa[r] = rows[rbase + srow + 64 * r];
-    asrc[r] = A + (int64_t)(GATED ? max(pa[r], 0) / top : rbase + srow + 64 * r) * lda + sch * 8;
+    asrc[r] = A + (int64_t)(FIRST ? max(pa[r], 0) / top : rbase + srow + 64 * r) * lda + sch * 8;
   }
   f32x4_t acc[MT][NT], accu[MT][NG];
 #pragma unroll
@@ -417,8 +437,10 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* 
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int rr = rbase + 16 * i + kg * 4 + r;
-        if (rows[rr] < 0) continue;
+        const int pr = rows[rr];
+        if (pr < 0) continue;
         if (GATED) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(glu(kind, acc[i][j][r], accu[i][GATED ? j : 0][r], limit, alpha));
+        else if (FIRST) ((bf16*)out)[(int64_t)rr * Nout + n] = f2bf(act1(kind, acc[i][j][r] * (row_scale ? row_scale[pr] : 1.f)));
         else ((float*)out)[(int64_t)rr * Nout + n] = acc[i][j][r];
       }
     }
@@ -429,7 +451,8 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const int32_t* _
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float acc = 0.f;
-    for (int j = 0; j < top; ++j) acc += wts[(int64_t)t * top + j] * y[(int64_t)dest[(int64_t)t * top + j] * W + c];
+    for (int j = 0; j < top; ++j)
+      acc += (wts ? wts[(int64_t)t * top + j] : 1.f) * y[(int64_t)dest[(int64_t)t * top + j] * W + c];
     out[(int64_t)t * W + c] = acc;
   }
 }
@@ -462,39 +485,40 @@ int moe_align(const int32_t* ids, int pairs, int E, int cap, int tm, int32_t* ro
 }
 
 int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int32_t* rows, const int32_t* tile_expert,
-                 int cap, int tm, int top, int Nout, int K, bool gated, void* out, int kind, float limit, float alpha,
-                 bool mfma, hipStream_t st) {
+                 int cap, int tm, int top, int Nout, int K, int mode, void* out, int kind, float limit, float alpha,
+                 const float* row_scale, bool mfma, hipStream_t st) {
   if (cap <= 0) return 0;
-  if ((tm != 16 && tm != 64 && tm != 128) || cap % tm != 0 || Nout < 1 || K < 1) return -1;
+  if ((tm != 16 && tm != 64 && tm != 128) || cap % tm != 0 || Nout < 1 || K < 1 || mode < kGemmRows || mode > kGemmAct ||
+      (mode == kGemmGated && kind != kGluGeluTanh && kind != kGluClamped) || (mode == kGemmAct && kind != kActRelu2) ||
+      (row_scale && mode != kGemmAct))
+    return -1;
   if (!f32 && mfma && K % 32 == 0 && Nout % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)Wt % 16 == 0) {
-#define XGM_GG(GATED, K64)                                                                                          \
-  grouped_gemm_mfma_kernel<GATED, 1, 2, true, K64><<<dim3(cap / tm, (Nout + 31) / 32), 256, 0, st>>>(                \
-      (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha);
-#define XGM_GL(GATED, MT, NT)                                                                                         \
-  grouped_gemm_mfma_lds_kernel<GATED, MT, NT><<<dim3(cap / (16 * MT), (Nout + 64 * NT - 1) / (64 * NT)), 256, 0, st>>>( \
-      (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, tm, top, Nout, K, out, kind, limit, alpha);
-    if (tm == 128) {         // gated: 64 x 128 per workgroup (two accumulator sets); plain: 128 x 128
-      if (gated) { XGM_GL(true, 4, 2) } else { XGM_GL(false, 8, 2) }
-    } else if (tm == 64) {   // gated: 64 x 128; plain: 64 x 256
-      if (gated) { XGM_GL(true, 4, 2) } else { XGM_GL(false, 4, 4) }
+#define XGM_GG(MODE, K64)                                                                                           \
+  grouped_gemm_mfma_kernel<MODE, 1, 2, true, K64><<<dim3(cap / tm, (Nout + 31) / 32), 256, 0, st>>>(                 \
+      (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha, row_scale);
+#define XGM_GL(MODE, MT, NT)                                                                                          \
+  grouped_gemm_mfma_lds_kernel<MODE, MT, NT><<<dim3(cap / (16 * MT), (Nout + 64 * NT - 1) / (64 * NT)), 256, 0, st>>>( \
+      (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, tm, top, Nout, K, out, kind, limit, alpha, row_scale);
+    if (tm == 128) {         // gated: 64 x 128 per workgroup (two accumulator sets); one weight block: 128 x 128
+      if (mode == kGemmGated) { XGM_GL(kGemmGated, 4, 2) } else if (mode == kGemmAct) { XGM_GL(kGemmAct, 8, 2) } else { XGM_GL(kGemmRows, 8, 2) }
+    } else if (tm == 64) {   // gated: 64 x 128; one weight block: 64 x 256
+      if (mode == kGemmGated) { XGM_GL(kGemmGated, 4, 2) } else if (mode == kGemmAct) { XGM_GL(kGemmAct, 4, 4) } else { XGM_GL(kGemmRows, 4, 4) }
     } else if (K % 64 == 0) {
-      if (gated) { XGM_GG(true, true) } else { XGM_GG(false, true) }
+      if (mode == kGemmGated) { XGM_GG(kGemmGated, true) } else if (mode == kGemmAct) { XGM_GG(kGemmAct, true) } else { XGM_GG(kGemmRows, true) }
     } else {
-      if (gated) { XGM_GG(true, false) } else { XGM_GG(false, false) }
+      if (mode == kGemmGated) { XGM_GG(kGemmGated, false) } else if (mode == kGemmAct) { XGM_GG(kGemmAct, false) } else { XGM_GG(kGemmRows, false) }
     }
 #undef XGM_GL
 #undef XGM_GG
     return 0;
   }
   dim3 grid(cap / 16, (Nout + 63) / 64);
-  if (gated) {
-    XGM_DISPATCH_T(f32, grouped_gemm_kernel<T, true><<<grid, 256, 0, st>>>((const T*)A, lda, (const T*)Wt, rows, tile_expert,
-                                                                            tm, top, Nout, K, out, kind, limit, alpha);)
-  } else {
-    XGM_DISPATCH_T(f32, grouped_gemm_kernel<T, false><<<grid, 256, 0, st>>>((const T*)A, lda, (const T*)Wt, rows,
-                                                                             tile_expert, tm, top, Nout, K, out, kind,
-                                                                             limit, alpha);)
-  }
+#define XGM_G0(MODE)                                                                                                    \
+  XGM_DISPATCH_T(f32, grouped_gemm_kernel<T, MODE><<<grid, 256, 0, st>>>((const T*)A, lda, (const T*)Wt, rows, tile_expert, \
+                                                                          tm, top, Nout, K, out, kind, limit, alpha,     \
+                                                                          row_scale);)
+  if (mode == kGemmGated) { XGM_G0(kGemmGated) } else if (mode == kGemmAct) { XGM_G0(kGemmAct) } else { XGM_G0(kGemmRows) }
+#undef XGM_G0
   return 0;
 }
 

@@ -14,20 +14,21 @@ void embed_rows(const int32_t*, const void*, bool, float*, int, int, int, const 
                 hipStream_t);
 void causal_conv(const void*, bool, int64_t, const float*, const float*, float*, const int32_t*, const int32_t*,
                  const int32_t*, void*, bool, int, int, int, int, bool, bool, hipStream_t);
-void residual_norm(float*, const void*, int64_t, const float*, const void*, int64_t, const float*, const float*, bool,
-                   const float*, float, float*, void*, bool, int, int, hipStream_t);
+int residual_norm(float*, const void*, int64_t, const float*, const void*, int64_t, const float*, const float*, bool,
+                  const float*, float, float*, void*, bool, int, int, int, const float*, const float*, hipStream_t);
 void qk_norm_cache(const void*, bool, int64_t, int, int, int, const float*, const float*, float, const int32_t*, void*,
                    void*, void*, int, hipStream_t);
 int masked_attention(const void*, bool, const void*, const void*, const int32_t*, int, int, const int32_t*,
                      const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
-                     const void*, int64_t, const float*, const float*, int, hipStream_t);
+                     const void*, int64_t, const float*, const float*, int, bool, int, const float*, hipStream_t);
 int masked_attention_mfma(const void*, const void*, const void*, const int32_t*, int, int, const int32_t*, const int32_t*,
                           const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, int, int,
-                          float, int, float*, float*, const void*, int64_t, const float*, const float*, int, int,
-                          hipStream_t);
+                          float, int, float*, float*, const void*, int64_t, const float*, const float*, int, int, bool, int,
+                          const float*, hipStream_t);
 void talk_mix(const void*, bool, const float*, const void*, int64_t, void*, int, int, int, int, hipStream_t);
 void head_norm_rope_cache(const void*, bool, int64_t, int, int, int, int, const float*, const float*, float, const float*,
-                          int, int, const int32_t*, const int32_t*, void*, void*, void*, bool, int, hipStream_t);
+                          int, int, const int32_t*, const int32_t*, void*, void*, void*, bool, int, bool, bool, const void*,
+                          int64_t, const float*, hipStream_t);
 int conv_head_norm_rope_cache(const void*, bool, int64_t, const float*, int, float*, const int32_t*, const int32_t*,
                               const int32_t*, const int32_t*, int, int, int, int, int, int, const float*, const float*,
                               float, const float*, int, int, const int32_t*, void*, void*, void*, bool, int, hipStream_t);
@@ -41,13 +42,17 @@ int gated_linear_scan(const float*, const float*, const float*, const void*, int
                       int, int, int, hipStream_t);
 int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, const float*, const float*, float*,
              const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, int, int, hipStream_t);
-void gated_group_norm(const float*, const void*, bool, int64_t, const float*, int, float, void*, int, int, int,
+void gated_group_norm(const float*, const void*, bool, int64_t, const float*, int, float, void*, int, int, int, bool,
                       hipStream_t);
 void glu_act(const void*, bool, int64_t, void*, int, int, int, float, float, hipStream_t);
 int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, hipStream_t);
 int moe_align(const int32_t*, int, int, int, int, int32_t*, int32_t*, int32_t*, hipStream_t);
-int grouped_gemm(const void*, bool, int64_t, const void*, const int32_t*, const int32_t*, int, int, int, int, int, bool, void*,
-                 int, float, float, bool, hipStream_t);
+int grouped_gemm(const void*, bool, int64_t, const void*, const int32_t*, const int32_t*, int, int, int, int, int, int, void*,
+                 int, float, float, const float*, bool, hipStream_t);
+int mingru_scan(const void*, bool, int64_t, int, int, int, int, const float*, const float*, float*, const int32_t*,
+                const int32_t*, const int32_t*, void*, bool, int, int, hipStream_t);
+void decay_gates(const void*, bool, int64_t, int, int, int, float, const void*, int64_t, const float*, float, float*, float*,
+                 float*, int, hipStream_t);
 void moe_combine(const float*, const int32_t*, const float*, int, int, int, float*, hipStream_t);
 void canon_conv(const float*, const float*, float*, const int32_t*, const int32_t*, const int32_t*, void*, bool, int, int,
                 int, int, hipStream_t);
@@ -98,12 +103,12 @@ PYBIND11_MODULE(_mixers, m) {
   });
   m.def("residual_norm", [](uintptr_t x, uintptr_t y1, int64_t ld1, uintptr_t a1, uintptr_t y2, int64_t ld2, uintptr_t y3,
                             uintptr_t a2, bool y_f32, uintptr_t g, float eps, uintptr_t n32, uintptr_t nact,
-                            bool nact_f32, int T, int W, uintptr_t st) {
+                            bool nact_f32, int T, int W, int groups, uintptr_t bw1, uintptr_t bw2, uintptr_t st) {
     if ((y1 && ld1 < W) || (y2 && ld2 < W)) throw std::invalid_argument("residual_norm: row stride smaller than the width");
-    xgm::residual_norm(P<float>(x), P<const void>(y1), ld1, P<const float>(a1), P<const void>(y2), ld2, P<const float>(y3),
-                       P<const float>(a2), y_f32, P<const float>(g), eps, P<float>(n32), P<void>(nact), nact_f32, T, W,
-                       S(st));
-    check(0, "residual_norm");
+    int rc = xgm::residual_norm(P<float>(x), P<const void>(y1), ld1, P<const float>(a1), P<const void>(y2), ld2,
+                                P<const float>(y3), P<const float>(a2), y_f32, P<const float>(g), eps, P<float>(n32),
+                                P<void>(nact), nact_f32, T, W, groups, P<const float>(bw1), P<const float>(bw2), S(st));
+    check(rc, "residual_norm");
   });
   m.def("qk_norm_cache", [](uintptr_t proj, bool f32, int64_t ld, int nq, int nk, int nv, uintptr_t wq, uintptr_t wk,
                             float eps, uintptr_t slot_mapping, uintptr_t q_out, uintptr_t kcache, uintptr_t vcache, int T,
@@ -116,13 +121,15 @@ PYBIND11_MODULE(_mixers, m) {
   m.def("masked_attention", [](uintptr_t q, bool f32, uintptr_t kc, uintptr_t vc, uintptr_t bt, int bt_width, int bs,
                                uintptr_t pos, uintptr_t token_seq, uintptr_t temp, uintptr_t sink, uintptr_t out, int T,
                                int H, int G, int dk, int dv, int mask, int size, float scale, uintptr_t gate,
-                               int64_t ld_gate, uintptr_t r1, uintptr_t r2, int vmode, uintptr_t st) {
-    if (bs < 1 || bt_width < 1 || (gate && ld_gate < H))
+                               int64_t ld_gate, uintptr_t r1, uintptr_t r2, int vmode, bool gate_elem, int wfn,
+                               uintptr_t hbias, uintptr_t st) {
+    if (bs < 1 || bt_width < 1 || (gate && ld_gate < (gate_elem ? (int64_t)H * dv : H)))
       throw std::invalid_argument("masked_attention: inconsistent sizes");
     int rc = xgm::masked_attention(P<const void>(q), f32, P<const void>(kc), P<const void>(vc), P<const int32_t>(bt),
                                    bt_width, bs, P<const int32_t>(pos), P<const int32_t>(token_seq), P<const float>(temp),
                                    P<const float>(sink), P<void>(out), T, H, G, dk, dv, mask, size, scale,
-                                   P<const void>(gate), ld_gate, P<const float>(r1), P<const float>(r2), vmode, S(st));
+                                   P<const void>(gate), ld_gate, P<const float>(r1), P<const float>(r2), vmode, gate_elem,
+                                   wfn, P<const float>(hbias), S(st));
     check(rc, "masked_attention");
   });
   m.def("masked_attention_mfma", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int bt_width, int bs,
@@ -130,15 +137,15 @@ PYBIND11_MODULE(_mixers, m) {
                                     uintptr_t out, int T, int ns, int max_q, int H, int G, int dk, int dv, int mask,
                                     int size, float scale, int nsplit, uintptr_t part_o, uintptr_t part_ml,
                                     uintptr_t gate, int64_t ld_gate, uintptr_t r1, uintptr_t r2, int vmode, int nw_hint,
-                                    uintptr_t st) {
-    if (bs < 1 || bt_width < 1 || nsplit < 1 || (gate && ld_gate < H))
+                                    bool gate_elem, int wfn, uintptr_t hbias, uintptr_t st) {
+    if (bs < 1 || bt_width < 1 || nsplit < 1 || (gate && ld_gate < (gate_elem ? (int64_t)H * dv : H)))
       throw std::invalid_argument("masked_attention_mfma: inconsistent sizes");
     int rc = xgm::masked_attention_mfma(P<const void>(q), P<const void>(kc), P<const void>(vc), P<const int32_t>(bt),
                                         bt_width, bs, P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
                                         P<const float>(temp), P<const float>(sink), P<void>(out), T, ns, max_q, H, G, dk,
                                         dv, mask, size, scale, nsplit, P<float>(part_o), P<float>(part_ml),
                                         P<const void>(gate), ld_gate, P<const float>(r1), P<const float>(r2), vmode,
-                                        nw_hint, S(st));
+                                        nw_hint, gate_elem, wfn, P<const float>(hbias), S(st));
     check(rc, "masked_attention_mfma");
   });
   m.def("talk_mix", [](uintptr_t o_all, bool f32, uintptr_t talk, uintptr_t gate, int64_t ld_gate, uintptr_t out, int T,
@@ -152,13 +159,15 @@ PYBIND11_MODULE(_mixers, m) {
   m.def("head_norm_rope_cache", [](uintptr_t src, bool src_f32, int64_t ld, int H, int G, int dk, int dv, uintptr_t wq,
                                    uintptr_t wk, float eps, uintptr_t rot, int rot_rows, int rot_dims, uintptr_t pos,
                                    uintptr_t slot_mapping, uintptr_t q_out, uintptr_t kc, uintptr_t vc, bool out_f32, int T,
-                                   uintptr_t st) {
+                                   bool whole, bool half, uintptr_t v_first, int64_t ld_vf, uintptr_t v_mix, uintptr_t st) {
     if (H < 1 || G < 1 || dk < 1 || dv < 1 || ld < (int64_t)(H + G) * dk + (int64_t)G * dv || rot_dims < 0 ||
-        rot_dims > dk || (rot_dims & 1) || (rot && rot_dims > 0 && rot_rows < 1))
+        rot_dims > dk || (rot_dims & 1) || (rot && rot_dims > 0 && rot_rows < 1) ||
+        (v_first && (!v_mix || ld_vf < (int64_t)G * dv)))
       throw std::invalid_argument("head_norm_rope_cache: inconsistent sizes");
     xgm::head_norm_rope_cache(P<const void>(src), src_f32, ld, H, G, dk, dv, P<const float>(wq), P<const float>(wk), eps,
                               P<const float>(rot), rot_rows, rot_dims, P<const int32_t>(pos),
-                              P<const int32_t>(slot_mapping), P<void>(q_out), P<void>(kc), P<void>(vc), out_f32, T, S(st));
+                              P<const int32_t>(slot_mapping), P<void>(q_out), P<void>(kc), P<void>(vc), out_f32, T, whole, half,
+                              P<const void>(v_first), ld_vf, P<const float>(v_mix), S(st));
     check(0, "head_norm_rope_cache");
   });
   m.def("conv_head_norm_rope_cache", [](uintptr_t proj, bool in_f32, int64_t ld, uintptr_t conv_w, int taps,
@@ -224,11 +233,11 @@ PYBIND11_MODULE(_mixers, m) {
     check(rc, "ssm_scan");
   });
   m.def("gated_group_norm", [](uintptr_t y, uintptr_t z, bool f32, int64_t ld_z, uintptr_t w, int wn, float eps,
-                               uintptr_t out, int T, int inner, int ng, uintptr_t st) {
+                               uintptr_t out, int T, int inner, int ng, bool gate_after, uintptr_t st) {
     if (ng < 1 || inner % ng || wn < 1 || inner % wn)
       throw std::invalid_argument("gated_group_norm: the parts and the weight's period must divide the row");
     xgm::gated_group_norm(P<const float>(y), P<const void>(z), f32, ld_z, P<const float>(w), wn, eps, P<void>(out), T,
-                          inner, ng, S(st));
+                          inner, ng, gate_after, S(st));
     check(0, "gated_group_norm");
   });
   m.def("glu_act", [](uintptr_t in, bool f32, int64_t ld, uintptr_t out, int T, int F, int kind, float limit, float alpha,
@@ -250,17 +259,37 @@ PYBIND11_MODULE(_mixers, m) {
     check(rc, "moe_align");
   });
   m.def("grouped_gemm", [](uintptr_t A, bool f32, int64_t lda, uintptr_t Wt, uintptr_t rows, uintptr_t tile_expert, int cap,
-                           int tm, int top, int Nout, int K, bool gated, uintptr_t out, int kind, float limit, float alpha,
-                           bool mfma, uintptr_t st) {
+                           int tm, int top, int Nout, int K, int mode, uintptr_t out, int kind, float limit, float alpha,
+                           uintptr_t row_scale, bool mfma, uintptr_t st) {
     if (top < 1 || lda < K) throw std::invalid_argument("grouped_gemm: inconsistent sizes");
     int rc = xgm::grouped_gemm(P<const void>(A), f32, lda, P<const void>(Wt), P<const int32_t>(rows),
-                               P<const int32_t>(tile_expert), cap, tm, top, Nout, K, gated, P<void>(out), kind, limit, alpha,
-                               mfma, S(st));
+                               P<const int32_t>(tile_expert), cap, tm, top, Nout, K, mode, P<void>(out), kind, limit, alpha,
+                               P<const float>(row_scale), mfma, S(st));
     check(rc, "grouped_gemm");
   });
   m.def("moe_combine", [](uintptr_t y, uintptr_t dest, uintptr_t wts, int T, int top, int W, uintptr_t out, uintptr_t st) {
     xgm::moe_combine(P<const float>(y), P<const int32_t>(dest), P<const float>(wts), T, top, W, P<float>(out), S(st));
     check(0, "moe_combine");
+  });
+
+  m.def("mingru_scan", [](uintptr_t proj, bool f32, int64_t ld, int off_z, int off_x, int off_g, int n, uintptr_t bz,
+                          uintptr_t bx, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t out,
+                          bool out_f32, int ns, int max_q, uintptr_t st) {
+    if (n < 1 || off_z < 0 || off_x < 0 || off_g < 0 || ld < off_z + n || ld < off_x + n || ld < off_g + n || !state)
+      throw std::invalid_argument("mingru_scan: columns outside the row");
+    int rc = xgm::mingru_scan(P<const void>(proj), f32, ld, off_z, off_x, off_g, n, P<const float>(bz), P<const float>(bx),
+                              P<float>(state), P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
+                              P<void>(out), out_f32, ns, max_q, S(st));
+    check(rc, "mingru_scan");
+  });
+  m.def("decay_gates", [](uintptr_t proj, bool f32, int64_t ld, int off_q, int off_k, int n, float q_scale, uintptr_t z,
+                          int64_t ld_z, uintptr_t zb, float inv_tau, uintptr_t q, uintptr_t f, uintptr_t k, int T,
+                          uintptr_t st) {
+    if (n < 1 || off_q < 0 || off_k < 0 || ld < off_q + n || ld < off_k + n || ld_z < n || !(inv_tau > 0.f))
+      throw std::invalid_argument("decay_gates: inconsistent arguments");
+    xgm::decay_gates(P<const void>(proj), f32, ld, off_q, off_k, n, q_scale, P<const void>(z), ld_z, P<const float>(zb),
+                     inv_tau, P<float>(q), P<float>(f), P<float>(k), T, S(st));
+    check(0, "decay_gates");
   });
 
   m.def("canon_conv", [](uintptr_t x, uintptr_t w, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,

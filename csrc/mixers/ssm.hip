@@ -8,7 +8,8 @@
 //                     x / B / C are columns of one activation row [x (H P) | B (G N) | C (G N)] (already
 //                     through their short convolution and activation), dt_raw a column block of another.
 //   gated_group_norm  v = y * silu(z) (v = y without z);  each of `ng` equal parts of v divided by its own root
-//                     mean square, times w (gated first, normed second); w repeats with period wn.
+//                     mean square, times w (gated first, normed second); w repeats with period wn. With
+//                     `gate_after` the norm is taken of y itself and silu(z) multiplies the normed, weighted result.
 //
 // One workgroup = (sequence, head, 64 state columns), NW waves: lane p owns column p, wave w owns rows
 // [w * NI, (w + 1) * NI) of it in registers (state rows are read and written 256 bytes at a time). B / C / x /
@@ -134,20 +135,24 @@ __global__ __launch_bounds__(64 * NW) void ssm_scan_kernel(const T* __restrict__
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z,
                                                                int64_t ld_z, const float* __restrict__ w, int wn,
-                                                               float eps, T* __restrict__ out, int inner, int gs) {
+                                                               float eps, T* __restrict__ out, int inner, int gs,
+                                                               int gate_after) {
   __shared__ float red[4];
   const int t = blockIdx.x, c0 = blockIdx.y * gs;
+  const bool pre = z && !gate_after, post = z && gate_after;
   float ss = 0.f;
   for (int c = threadIdx.x; c < gs; c += blockDim.x) {
     float v = y[(int64_t)t * inner + c0 + c];
-    if (z) v *= siluf(ldf(z + (int64_t)t * ld_z + c0 + c));
+    if (pre) v *= siluf(ldf(z + (int64_t)t * ld_z + c0 + c));
     ss += v * v;
   }
   const float r = 1.f / sqrtf(block_sum(ss, red) / (float)gs + eps);
   for (int c = threadIdx.x; c < gs; c += blockDim.x) {
     float v = y[(int64_t)t * inner + c0 + c];
-    if (z) v *= siluf(ldf(z + (int64_t)t * ld_z + c0 + c));
-    stf(out + (int64_t)t * inner + c0 + c, v * r * w[(c0 + c) % wn]);
+    if (pre) v *= siluf(ldf(z + (int64_t)t * ld_z + c0 + c));
+    v = v * r * w[(c0 + c) % wn];
+    if (post) v *= siluf(ldf(z + (int64_t)t * ld_z + c0 + c));
+    stf(out + (int64_t)t * inner + c0 + c, v);
   }
 }
 
@@ -172,12 +177,12 @@ int ssm_scan(const void* xbc, bool f32, int64_t ld_x, const void* dt_raw, int64_
 }
 
 void gated_group_norm(const float* y, const void* z, bool f32, int64_t ld_z, const float* w, int wn, float eps, void* out,
-                      int T_, int inner, int ng, hipStream_t st) {
+                      int T_, int inner, int ng, bool gate_after, hipStream_t st) {
   if (T_ <= 0) return;
   // small groups (one per head): fewer threads per group
   const int gs = inner / ng, nth = gs <= 64 ? 64 : gs <= 128 ? 128 : 256;
   XGM_DISPATCH_T(f32, gated_group_norm_kernel<T><<<dim3(T_, ng), nth, 0, st>>>(y, (const T*)z, ld_z, w, wn, eps, (T*)out,
-                                                                                inner, gs);)
+                                                                                inner, gs, gate_after ? 1 : 0);)
 }
 
 }  // namespace xgm

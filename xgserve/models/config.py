@@ -16,7 +16,7 @@ from typing import Dict, List, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" | "mixtral" | "gpt2" | "dofivik" | "vizonex" | "loluzen"
+    arch: str                      # "llama" | "mixtral" | "gpt2" | "dofivik" | "vizonex" | "loluzen" | "lotelix"
     hidden_size: int
     num_layers: int
     num_heads: int
@@ -44,6 +44,8 @@ class ModelConfig:
     embed_scale: float = 1.0
     residual_mult: float = 1.0
     layer_loop: Optional[dict] = None
+    # "lotelix": the equal consecutive parts of a row that its RMS norms treat separately
+    norm_groups: int = 1
 
     @property
     def q_size(self) -> int:
@@ -60,6 +62,8 @@ class ModelConfig:
                 from .vizonex import count_params
             elif self.arch == "loluzen":
                 from .loluzen import count_params
+            elif self.arch == "lotelix":
+                from .lotelix import count_params
             else:
                 from .dofivik import count_params
             return count_params(self)
@@ -85,6 +89,9 @@ class ModelConfig:
     def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
         if self.arch == "loluzen":
             att = [(m.get("left") or m) for m in (self.layer_specs[i]["mixer"] for i in self.layer_runs())]
+            return sum((m["dim"] + m["vdim"]) * m["kv_heads"] * dtype_bytes for m in att)
+        if self.arch == "lotelix":
+            att = [(L["mixer"].get("left") or L["mixer"]) for L in self.layer_specs if L["type"] != "mingru"]
             return sum((m["dim"] + m["vdim"]) * m["kv_heads"] * dtype_bytes for m in att)
         if self.arch == "vizonex":
             return sum((m["dim"] + m["vdim"]) * m["kv_heads"] * dtype_bytes
@@ -302,6 +309,90 @@ def _loluzen_tiny_layers():
 
 register(loluzen_config("loluzen-tiny", 128, 512, _loluzen_tiny_layers(), embed_scale=4.0, residual_mult=0.5,
                         loop={"start": 1, "stop": 2, "times": 2}, max_position=1024))
+def lotelix_config(name: str, width: int, vocab: int, layers: List[dict], embed_scale: float = 1.0, eps: float = 1e-5,
+                   norm_groups: int = 1, max_position: int = 131072) -> ModelConfig:
+    """A Lotelix model: pre-norm layers x <- x + mixer(N(x)), x <- x + ff(N(x)) whose RMS norm N treats `norm_groups`
+    equal consecutive parts of a row separately. Mixers: "mingru" (a per-channel gated recurrence whose gate and
+    candidate read the current token only), "attention" (rotation in (i, i + dims / 2) pairs with rescaled
+    frequencies, sliding window, softmax sink, values blended with the first value-mixing layer's, element-wise output
+    gate) and "parallel" (causal attention with unnormalised sigmoid weights, biased projections and whole-vector
+    q / k norms beside a linear attention with a decay per key channel). Feed-forward: a sigmoid-routed mixture of
+    squared-relu experts whose routing weight scales the expert's input, or none."""
+    def need(d, keys, where):
+        for k in keys:
+            if k not in d:
+                raise ValueError(f"{where}: missing {k!r}")
+
+    def gqa(m, w):
+        need(m, ("heads", "kv_heads", "dim", "vdim", "scale"), w)
+        if m["heads"] < 1 or m["kv_heads"] < 1 or m["heads"] % m["kv_heads"]:
+            raise ValueError(f"{w}: heads must be a positive multiple of kv_heads")
+        rot = m.get("rot")
+        if rot is not None:
+            need(rot, ("base", "dims"), w)
+            if rot["dims"] % 2 or not 0 <= rot["dims"] <= m["dim"]:
+                raise ValueError(f"{w}: rot.dims must be even and at most dim")
+            if rot.get("scaling") is not None:
+                need(rot["scaling"], ("factor", "low", "high", "original"), w)
+    if not layers:
+        raise ValueError("a model needs at least one layer")
+    if norm_groups < 1 or norm_groups > 64 or width % norm_groups:
+        raise ValueError("norm.groups must be in [1, 64] and divide the width")
+    mixed = None
+    for i, L in enumerate(layers):
+        m, w = L.get("mixer") or {}, f"layer {i}"
+        if L.get("type") == "mingru":
+            need(m, ("width",), w)
+            if m["width"] < 1:
+                raise ValueError(f"{w}: width must be positive")
+        elif L.get("type") == "attention":
+            gqa(m, w)
+            if m.get("mask") is not None and int(m["mask"]["size"]) < 1:
+                raise ValueError(f"{w}: mask.size must be positive")
+            if m.get("v_mix"):
+                if mixed is not None and mixed != m["kv_heads"] * m["vdim"]:
+                    raise ValueError(f"{w}: value-mixing layers must have value rows of equal size")
+                mixed = m["kv_heads"] * m["vdim"]
+        elif L.get("type") == "parallel":
+            need(m, ("left", "right"), w)
+            gqa(m["left"], w + " left")
+            need(m["right"], ("heads", "dim", "vdim", "tau"), w + " right")
+            if m["right"]["dim"] > 256 or m["right"]["tau"] <= 0:
+                raise ValueError(f"{w}: recurrent head sizes above 256 are not supported; tau must be positive")
+        else:
+            raise ValueError(f"{w}: unknown mixer type {L.get('type')!r}")
+        mlp = L.get("mlp")
+        if mlp is not None:
+            if mlp.get("kind") != "moe":
+                raise ValueError(f"{w}: unknown feed-forward kind {mlp.get('kind')!r}")
+            need(mlp, ("expert", "router"), w)
+            need(mlp["router"], ("experts", "top"), w)
+            need(mlp["expert"], ("ff",), w)
+            if not 1 <= mlp["router"]["top"] <= mlp["router"]["experts"] <= 512:
+                raise ValueError(f"{w}: needs 1 <= top <= experts <= 512")
+    att = [(L["mixer"].get("left") or L["mixer"]) for L in layers if L["type"] != "mingru"]
+    heads = max([m["heads"] for m in att] or [1])
+    hd = max([max(m["dim"], m["vdim"]) for m in att] or [1])
+    ff = max([L["mlp"]["expert"]["ff"] * L["mlp"]["router"]["top"] for L in layers if L.get("mlp")] or [0])
+    return ModelConfig(name, "lotelix", width, len(layers), heads, max([m["kv_heads"] for m in att] or [1]), hd, ff, vocab,
+                       max_position, 0.0, None, eps, False, bos_token_id=0, eos_token_ids=[], layer_specs=layers,
+                       embed_scale=float(embed_scale), norm_groups=int(norm_groups))
+
+
+def _lotelix_tiny_layers():
+    att = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.2, "mask": {"size": 24}, "v_mix": True,
+           "rot": {"base": 10000.0, "dims": 16, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}}}
+    par = {"left": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.25, "rot": {"base": 5000.0, "dims": 8}},
+           "right": {"heads": 2, "dim": 16, "vdim": 32, "tau": 8.0, "decay_rank": 8}}
+    moe = {"kind": "moe", "expert": {"ff": 48}, "router": {"experts": 6, "top": 2}}
+    return [{"type": "attention", "mixer": dict(att), "mlp": dict(moe)},
+            {"type": "mingru", "mixer": {"width": 96}, "mlp": None},
+            {"type": "parallel", "mixer": par, "mlp": dict(moe)},
+            {"type": "attention", "mixer": dict(att), "mlp": dict(moe)}]
+
+
+register(lotelix_config("lotelix-tiny", 128, 512, _lotelix_tiny_layers(), embed_scale=3.0, norm_groups=4,
+                        max_position=1024))
 register(ModelConfig("gpt2-tiny", "gpt2", 128, 2, 2, 2, 64, 512, 512, 256, 0.0, tie_embeddings=True,
                      bos_token_id=0, eos_token_ids=[0], dtype="float32"))
 
@@ -330,6 +421,9 @@ def from_hf_config(path: str, name: Optional[str] = None) -> ModelConfig:
     if c.get("architecture") == "Loluzen":
         return loluzen_config(name or "loluzen", c["width"], c["vocab"], c["layers"], c["embedding"]["scale"],
                               c["residual_mult"], c.get("loop"), c["norm"]["eps"], int(c.get("max_position", 131072)))
+    if c.get("architecture") == "Lotelix":
+        return lotelix_config(name or "lotelix", c["width"], c["vocab"], c["layers"], c["embedding"]["scale"],
+                              c["norm"]["eps"], int(c["norm"].get("groups", 1)), int(c.get("max_position", 131072)))
     mt = c.get("model_type", "llama")
     eos = c.get("eos_token_id", 2)
     eos = eos if isinstance(eos, list) else [eos]

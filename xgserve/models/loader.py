@@ -23,17 +23,24 @@ from .dofivik import DofivikForCausalLM
 from .gpt2 import GPT2ForCausalLM
 from .llama import LlamaForCausalLM
 from .loluzen import LoluzenForCausalLM
+from .lotelix import LotelixForCausalLM
 from .vizonex import VizonexForCausalLM
 
 
 def model_class(cfg: ModelConfig):
     return {"gpt2": GPT2ForCausalLM, "dofivik": DofivikForCausalLM, "vizonex": VizonexForCausalLM,
-            "loluzen": LoluzenForCausalLM}.get(cfg.arch, LlamaForCausalLM)
+            "loluzen": LoluzenForCausalLM, "lotelix": LotelixForCausalLM}.get(cfg.arch, LlamaForCausalLM)
 
 
 def _resolve_shapes(cfg: ModelConfig, checkpoint: str) -> None:
     """Sizes that only a tensor's shape gives (Dofivik: the rank of the decay projection; Loluzen: the taps of
-    a short convolution when the configuration leaves them out)."""
+    a short convolution when the configuration leaves them out; Lotelix: the rank of the decay projection)."""
+    if cfg.arch == "lotelix":
+        r = _Reader(checkpoint)
+        for i, spec in enumerate(cfg.layer_specs):
+            if spec["type"] == "parallel":
+                spec["mixer"]["right"]["decay_rank"] = int(r.shape(f"l{i}.mix.right.a1")[0])
+        return
     if cfg.arch == "loluzen":
         r = _Reader(checkpoint)
         for i, spec in enumerate(cfg.layer_specs):
@@ -106,9 +113,9 @@ class _Reader:
     def get(self, name: str, dim: Optional[int] = None, start: int = 0, length: Optional[int] = None) -> torch.Tensor:
         if name not in self.where:
             raise KeyError(f"missing tensor {name!r} in checkpoint {self.path}")
-        sl = self.handles[self.where[name]].get_slice(name)
         if dim is None:
-            return sl[:]
+            return self.handles[self.where[name]].get_tensor(name)   # (also a tensor without dimensions)
+        sl = self.handles[self.where[name]].get_slice(name)
         shape = sl.get_shape()
         end = start + (length if length is not None else shape[dim] - start)
         idx = [slice(None)] * len(shape)
@@ -134,6 +141,8 @@ def load_checkpoint(model, path: str) -> None:
         _load_vizonex(model, r)
     elif cfg.arch == "loluzen":
         _load_loluzen(model, r)
+    elif cfg.arch == "lotelix":
+        _load_lotelix(model, r)
     else:
         _load_llama(model, r)
 
@@ -352,6 +361,79 @@ def _save_loluzen(model, path: str) -> None:
                    "max_position": cfg.max_position}, f, indent=1)
 
 
+def _lotelix_tensors(m):
+    """(checkpoint name, parameter, index of a fused / stacked parameter or None) for every tensor."""
+    out = [("embed", m.embed, None), ("head", m.head, None), ("final.norm", m.final_norm, None)]
+    for i, L in enumerate(m.layers):
+        b, x = f"l{i}.", L.mix
+        out.append((b + "norm1", L.norm1, None))
+        if L.kind == "mingru":
+            n = x.n
+            out += [(b + "mix.z", x.in_proj, slice(0, n)), (b + "mix.x", x.in_proj, slice(n, 2 * n)),
+                    (b + "mix.g", x.in_proj, slice(2 * n, 3 * n)), (b + "mix.z.b", x.z_b, None),
+                    (b + "mix.x.b", x.x_b, None), (b + "mix.o", x.o, None)]
+        elif L.kind == "attention":
+            nq, nk = x.nq, x.nk
+            out += [(b + "mix.q", x.in_proj, slice(0, nq)), (b + "mix.k", x.in_proj, slice(nq, nq + nk)),
+                    (b + "mix.v", x.in_proj, slice(nq + nk, x.ch)), (b + "mix.g", x.in_proj, slice(x.ch, x.ch + x.H * x.dv)),
+                    (b + "mix.sink", x.sink, None), (b + "mix.o", x.o, None)]
+            if x.v_mix:
+                out.append((b + "mix.vmix", x.lam, "scalar"))
+        else:
+            a, r = x.left, x.right
+            at = 0
+            for name, rows, bias in (("left.q", a.nq, True), ("left.k", a.nk, True), ("left.v", a.nv, True),
+                                     ("right.q", r.n, False), ("right.k", r.n, False), ("right.v", r.nv, False),
+                                     ("right.g", r.nv, False), ("right.a1", r.rank, False)):
+                out.append((b + "mix." + name, x.in_proj, slice(at, at + rows)))
+                if bias:
+                    out.append((b + "mix." + name + ".b", x.in_bias, slice(at, at + rows)))
+                at += rows
+            out += [(b + "mix.left.q.norm", a.q_norm, None), (b + "mix.left.k.norm", a.k_norm, None),
+                    (b + "mix.left.pb", a.pb, None), (b + "mix.left.o", a.o, None), (b + "mix.left.o.b", a.o_b, None),
+                    (b + "mix.left.out", a.out_norm, None), (b + "mix.right.a2", r.a2, None),
+                    (b + "mix.right.a2.b", r.a2_b, None), (b + "mix.right.norm", r.norm, None),
+                    (b + "mix.right.o", r.o, None), (b + "mix.right.out", r.out_norm, None)]
+        if L.mlp is not None:
+            out += [(b + "norm2", L.norm2, None), (b + "mlp.router", L.mlp.router, None)]
+            for e in range(L.mlp.E):
+                out += [(f"{b}mlp.e{e}.up", L.mlp.up, e), (f"{b}mlp.e{e}.down", L.mlp.down, e)]
+    return out
+
+
+def _load_lotelix(m, r: _Reader):
+    """Tensors `embed`, `head`, `final.norm`, `l<i>.<norm1|norm2>`, `l<i>.mix.*`, `l<i>.mlp.*` ([out, in] matrices).
+    The projections that read the same input (and their biases) are fused row-wise, the experts stacked, on load."""
+    for name, p, idx in _lotelix_tensors(m):
+        src = r.get(name)
+        if idx == "scalar":
+            src, idx = src.reshape(1), None
+        dst = p.data if idx is None else p.data[idx]
+        if tuple(dst.shape) != tuple(src.shape):
+            raise ValueError(f"shape mismatch for {name}: model {tuple(dst.shape)} vs checkpoint {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+
+def _save_lotelix(model, path: str) -> None:
+    from safetensors.torch import save_file
+    cfg = model.cfg
+    t = {}
+    for name, p, idx in _lotelix_tensors(model):
+        v = p.data.reshape(()) if idx == "scalar" else p.data if idx is None else p.data[idx]
+        t[name] = v.detach().to(torch.bfloat16).contiguous().cpu()
+    save_file(t, os.path.join(path, "model.safetensors"))
+    layers = []
+    for spec in cfg.layer_specs:
+        mx = dict(spec["mixer"])
+        if spec["type"] == "parallel":   # the rank of the decay projection is given by a tensor's shape
+            mx["right"] = {k: v for k, v in mx["right"].items() if k != "decay_rank"}
+        layers.append({"type": spec["type"], "mixer": mx, "mlp": spec.get("mlp")})
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump({"architecture": "Lotelix", "width": cfg.hidden_size, "vocab": cfg.vocab_size,
+                   "embedding": {"scale": cfg.embed_scale}, "layers": layers,
+                   "norm": {"eps": cfg.norm_eps, "groups": cfg.norm_groups}, "max_position": cfg.max_position}, f, indent=1)
+
+
 def _save_vizonex(model, path: str) -> None:
     from safetensors.torch import save_file
     cfg = model.cfg
@@ -397,6 +479,8 @@ def save_checkpoint(model, path: str) -> None:
         return _save_vizonex(model, path)
     if cfg.arch == "loluzen":
         return _save_loluzen(model, path)
+    if cfg.arch == "lotelix":
+        return _save_lotelix(model, path)
     t: Dict[str, torch.Tensor] = {}
     if cfg.arch == "gpt2":
         t["transformer.wte.weight"] = model.wte

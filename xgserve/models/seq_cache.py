@@ -27,6 +27,7 @@ class LayerCache:
     mix_conv: Optional[torch.Tensor] = None  # a mixer's own short convolution: [slots, taps - 1, channels]
     ssm: Optional[torch.Tensor] = None      # state-space recurrence: [slots, heads, state, vdim]
     gla: Optional[torch.Tensor] = None      # gated linear recurrence: [slots, heads, dim, vdim]
+    gru: Optional[torch.Tensor] = None      # minimal gated recurrence: [slots, width]
 
 
 @dataclass

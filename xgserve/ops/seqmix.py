@@ -195,16 +195,18 @@ def build_rot_table(dims: int, base: float, max_pos: int, device="cpu", scaling:
     return torch.stack([ang.cos(), ang.sin()], -1).float().contiguous().to(device)
 
 
-def _rotate_pairs(v: torch.Tensor, rot: torch.Tensor, pos: torch.Tensor, dims: int) -> torch.Tensor:
-    """v [T, ..., n] fp32: rotate the first `dims` entries pairwise by the table rows of `pos`."""
+def _rotate_pairs(v: torch.Tensor, rot: torch.Tensor, pos: torch.Tensor, dims: int, half: bool = False) -> torch.Tensor:
+    """v [T, ..., n] fp32: rotate the first `dims` entries pairwise by the table rows of `pos`; pair i is entries
+    (2 i, 2 i + 1), or (i, i + dims / 2) with `half`."""
     cs = rot[pos.long()]  # [T, dims/2, 2]
     while cs.dim() < v.dim() + 1:
         cs = cs.unsqueeze(1)
     c, s = cs[..., 0], cs[..., 1]
-    a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+    ia, ib = (slice(0, dims // 2), slice(dims // 2, dims)) if half else (slice(0, dims, 2), slice(1, dims, 2))
+    a, b = v[..., ia], v[..., ib]
     out = v.clone()
-    out[..., 0:dims:2] = a * c - b * s
-    out[..., 1:dims:2] = b * c + a * s
+    out[..., ia] = a * c - b * s
+    out[..., ib] = b * c + a * s
     return out
 
 
@@ -400,23 +402,36 @@ def tanh_cols(x: torch.Tensor, off: int, n: int) -> torch.Tensor:
 # ---------------------------------------------------------------------------- parallel-block residual + next norm
 def residual_norm(x: torch.Tensor, y1: Optional[torch.Tensor], a1: Optional[torch.Tensor], y2: Optional[torch.Tensor],
                   y3: Optional[torch.Tensor], a2: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float,
-                  out_dtype: Optional[torch.dtype] = None, want_f32: bool = False):
+                  out_dtype: Optional[torch.dtype] = None, want_f32: bool = False, groups: int = 1,
+                  branch_w: Optional[tuple] = None):
     """x <- x + a1 * y1 + a2 * (y2 + y3) in place (x fp32 [T, W]; y1 / y2 activation tensors, y3 fp32; a1 / a2
     per-channel scales, None = 1; any y may be None), then, with `norm_w`, the RMS norm of the new x:
-    n = x / sqrt(mean(x^2) + eps) * norm_w, returned as (n fp32 or None, n as out_dtype or None)."""
+    n = x / sqrt(mean(x^2) + eps) * norm_w, returned as (n fp32 or None, n as out_dtype or None).
+    `groups` > 1: the norm splits a row into that many equal consecutive parts, each divided by its own root mean
+    square. `branch_w` = (w1, w2): y1 and y2 are the outputs of two branches that are averaged after each is
+    RMS-normed over the row with its plain weight, x <- x + (N0(y1) w1 + N0(y2) w2) / 2 + y3 (no a1 / a2)."""
     T, W = x.shape
+    assert groups >= 1 and W % groups == 0
     if not native_device(x):
+        def n0(v):
+            return v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
         v = x
-        if y1 is not None:
-            v = v + (a1 if a1 is not None else 1.0) * y1.float()
-        if y2 is not None or y3 is not None:
-            f = (y2.float() if y2 is not None else 0.0) + (y3 if y3 is not None else 0.0)
-            v = v + (a2 if a2 is not None else 1.0) * f
+        if branch_w is not None:
+            v = v + 0.5 * (n0(y1.float()) * branch_w[0] + n0(y2.float()) * branch_w[1])
+            if y3 is not None:
+                v = v + y3
+        else:
+            if y1 is not None:
+                v = v + (a1 if a1 is not None else 1.0) * y1.float()
+            if y2 is not None or y3 is not None:
+                f = (y2.float() if y2 is not None else 0.0) + (y3 if y3 is not None else 0.0)
+                v = v + (a2 if a2 is not None else 1.0) * f
         x.copy_(v)
         if norm_w is None:
             return None, None
-        n = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * norm_w
+        n = n0(x.view(T, groups, W // groups)).reshape(T, W) * norm_w
         return (n if want_f32 else None), (n.to(out_dtype) if out_dtype is not None else None)
+    assert branch_w is None or (y1 is not None and y2 is not None and a1 is None and a2 is None)
     assert x.dtype == torch.float32 and x.is_contiguous()
     ys = [y for y in (y1, y2) if y is not None]
     assert all(y.stride(1) == 1 and y.shape == x.shape for y in ys) and len({y.dtype for y in ys}) <= 1
@@ -426,6 +441,7 @@ def residual_norm(x: torch.Tensor, y1: Optional[torch.Tensor], a1: Optional[torc
     mixers().residual_norm(x.data_ptr(), _p(y1), y1.stride(0) if y1 is not None else 0, _p(a1), _p(y2),
                            y2.stride(0) if y2 is not None else 0, _p(y3), _p(a2), is_f32(ys[0]) if ys else True,
                            _p(norm_w), float(eps), _p(n32), _p(nact), is_f32(nact) if nact is not None else True, T, W,
+                           int(groups), _p(branch_w[0]) if branch_w else 0, _p(branch_w[1]) if branch_w else 0,
                            stream_ptr())
     return n32, nact
 
@@ -478,17 +494,22 @@ def qk_norm_cache(proj: torch.Tensor, nq: int, nk: int, nv: int, wq: Optional[to
 
 V_OWN, V_ALL = -1, -2   # masked_attention(values=...): the query head's own key/value head, or every head's values
 V_ALL_MAX = 256         # ... V_ALL serves up to this many value columns (G * dv) per query head
+W_SOFTMAX, W_SIGMOID = 0, 1   # masked_attention(weights=...): how scores become weights
 
 
 def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, H: int, G: int, dk: int, dv: int,
                      mask: int, size: int, scale: float, temp: Optional[torch.Tensor], sink: Optional[torch.Tensor],
                      block_size: int, sm: SeqMeta, gate: Optional[torch.Tensor] = None,
-                     dist: Optional[tuple] = None, values: int = V_OWN) -> torch.Tensor:
+                     dist: Optional[tuple] = None, values: int = V_OWN, gate_elem: bool = False,
+                     weights: int = W_SOFTMAX, score_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention of H query heads over G cached key/value heads (query head h reads head h // (H / G)).
     A query at position i sees keys first_visible(mask, size, i) .. i of its own sequence. score = (q . k) * scale
     * temp[h]; with `dist` = (r1, r2) (fp32 [H] each) the score of key j loses r1[h] * ln(1 + r2[h] * (i - j)),
     otherwise positions do not enter the scores; with `sink` the denominator also holds exp(sink[h]), a term with no
-    key and no value; with `gate` ([T, >= H], row-strided) head h's output is multiplied by sigmoid(gate[t, h]).
+    key and no value; with `gate` ([T, >= H], row-strided) head h's output is multiplied by sigmoid(gate[t, h]), or,
+    with `gate_elem` (gate [T, >= H dv]), entry d of head h by sigmoid(gate[t, h dv + d]).
+    `weights` = W_SIGMOID: no softmax; the weight of a visible key is sigmoid(score + score_bias[h]) (fp32 [H], None =
+    0), not normalised over the keys (no sink).
     `values`: V_OWN: head h weighs the values of its own key/value head, returns [T, H * dv]; V_ALL: the values of
     all G heads concatenated, returns [T, H * G * dv] (what mixing of the heads' weight maps needs);
     c >= 0: the values of head c for every query head.
@@ -499,7 +520,11 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
     if native_device(q):
         assert q.is_contiguous() and kcache.is_contiguous() and vcache.is_contiguous()
         assert kcache.dtype == vcache.dtype == q.dtype and -2 <= values < G
-        assert gate is None or (gate.stride(1) == 1 and gate.dtype == q.dtype and gate.shape[1] >= H)
+        assert gate is None or (gate.stride(1) == 1 and gate.dtype == q.dtype and
+                                gate.shape[1] >= (H * dv if gate_elem else H))
+        assert not gate_elem or values == V_OWN
+        assert weights == W_SOFTMAX or (sink is None and weights == W_SIGMOID)
+        assert score_bias is None or (score_bias.dtype == torch.float32 and score_bias.numel() == H)
         r1, r2 = dist if dist is not None else (None, None)
         bt = _i32(sm.block_tables)
         single = sm.max_q == 1 and T == sm.num_seqs
@@ -519,13 +544,14 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
                                            _i32(sm.slots).data_ptr(), _p(temp), _p(sink), out.data_ptr(), T, sm.num_seqs,
                                            sm.max_q, H, G, dk, dv, int(mask), int(size), float(scale), nsplit,
                                            _p(part_o), _p(part_ml), _p(gate), gate.stride(0) if gate is not None else 0,
-                                           _p(r1), _p(r2), int(values), ATTN_WAVES, stream_ptr())
+                                           _p(r1), _p(r2), int(values), ATTN_WAVES, bool(gate_elem), int(weights),
+                                           _p(score_bias), stream_ptr())
             return out
         mixers().masked_attention(q.data_ptr(), is_f32(q), kcache.data_ptr(), vcache.data_ptr(), bt.data_ptr(),
                                   bt.shape[1], block_size, _i32(sm.positions).data_ptr(), _i32(sm.token_seq).data_ptr(),
                                   _p(temp), _p(sink), out.data_ptr(), T, H, G, dk, dv, int(mask), int(size), float(scale),
                                   _p(gate), gate.stride(0) if gate is not None else 0, _p(r1), _p(r2), int(values),
-                                  stream_ptr())
+                                  bool(gate_elem), int(weights), _p(score_bias), stream_ptr())
         return out
     kr, vr = kcache.view(-1, G, dk), vcache.view(-1, G, dv)
     qf = q.float().view(T, H, dk)
@@ -543,16 +569,21 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         sc = torch.einsum("hd,nhd->hn", qf[t], kk) * (scale * tmp)[:, None]
         if dist is not None:
             sc = sc - dist[0][:, None] * torch.log1p(dist[1][:, None] * (pos[t] - keys).float()[None, :])
-        if sink is not None:
-            sc = torch.cat([sc, sink[:, None]], 1)
-        p = torch.softmax(sc, -1)[:, :keys.numel()]
+        if weights == W_SIGMOID:
+            p = torch.sigmoid(sc + (score_bias[:, None] if score_bias is not None else 0.0))
+        else:
+            if sink is not None:
+                sc = torch.cat([sc, sink[:, None]], 1)
+            p = torch.softmax(sc, -1)[:, :keys.numel()]
         if values == V_ALL:
             o = torch.einsum("hn,nd->hd", p, vr[idx].float().reshape(keys.numel(), G * dv))
         elif values >= 0:
             o = torch.einsum("hn,nd->hd", p, vr[idx][:, values].float())
         else:
             o = torch.einsum("hn,nhd->hd", p, vr[idx].float().repeat_interleave(rep, 1))
-        if gate is not None:
+        if gate is not None and gate_elem:
+            o = o * torch.sigmoid(gate[t, :H * dv].float()).view(H, dv)
+        elif gate is not None:
             o = o * torch.sigmoid(gate[t, :H].float())[:, None]
         out[t] = o.reshape(H * dvo).to(out.dtype)
     return out
@@ -594,30 +625,37 @@ def ssm_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A_l
 
 
 def gated_group_norm(y: torch.Tensor, z: Optional[torch.Tensor], w: torch.Tensor, eps: float, groups: int,
-                     out_dtype: torch.dtype) -> torch.Tensor:
+                     out_dtype: torch.dtype, gate_after: bool = False) -> torch.Tensor:
     """v = y * silu(z) (v = y when z is None); each of `groups` equal parts of a row divided by its own root mean
     square; times w, which holds one weight per column or one period of a repeating pattern (e.g. a weight of one
-    head's size shared by all heads). y fp32 [T, n]; z [T, n] (row-strided activation)."""
+    head's size shared by all heads). With `gate_after` the norm is taken of y itself and silu(z) multiplies the
+    normed, weighted result. y fp32 [T, n]; z [T, n] (row-strided activation)."""
     T, n = y.shape
     assert n % groups == 0 and n % w.numel() == 0
     if not native_device(y):
         v = y
+        gate = None
         if z is not None:
             zf = z.float()
-            v = y * zf * torch.sigmoid(zf)
+            gate = zf * torch.sigmoid(zf)
+            if not gate_after:
+                v = y * gate
         v = v.view(T, groups, n // groups)
-        v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, n)
-        return (v * w.repeat(n // w.numel())).to(out_dtype)
+        v = (v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, n) * w.repeat(n // w.numel())
+        if gate_after and gate is not None:
+            v = v * gate
+        return v.to(out_dtype)
     out = torch.empty(T, n, dtype=out_dtype, device=y.device)
     assert y.is_contiguous() and y.dtype == torch.float32 and w.dtype == torch.float32
     assert z is None or (z.stride(1) == 1 and z.dtype == out_dtype)
     mixers().gated_group_norm(y.data_ptr(), _p(z), is_f32(out), z.stride(0) if z is not None else 0, w.data_ptr(),
-                              w.numel(), float(eps), out.data_ptr(), T, n, groups, stream_ptr())
+                              w.numel(), float(eps), out.data_ptr(), T, n, groups, bool(gate_after), stream_ptr())
     return out
 
 
 # ---------------------------------------------------------------------------- gated feed-forward, routed experts
 GLU_GELU_TANH, GLU_CLAMPED = 0, 1
+ACT_RELU2 = 2   # routed_experts(kind=...): an expert without a gate, W_down relu(W_up h)^2
 # XGS_TUNE moe_mfma=0: the general grouped GEMM for bf16 too (A/B and tests)
 MOE_MFMA = tune.get_bool("moe_mfma", True)
 MOE_TILE_SMALL, MOE_TILES_BIG = 16, (128, 64)   # rows per expert tile of the sorted layout
@@ -672,13 +710,23 @@ def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], cou
     return ids, wts
 
 
+def _act_ref(z, kind):
+    assert kind == ACT_RELU2
+    return torch.relu(z).pow(2)
+
+
 def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, kind: int,
-                   limit: float, alpha: float = 1.702) -> torch.Tensor:
+                   limit: float = 0.0, alpha: float = 1.702, scale_input: bool = False) -> torch.Tensor:
     """sum_j wts[t, j] * W2[e] glu(W13[e] h_t), e = ids[t, j]. w13 [E, 2 F, K] holds each expert's gate rows then
-    its up rows, w2 [E, W, F]. Returns fp32 [T, W] (a sum in a fixed order per row)."""
+    its up rows, w2 [E, W, F]. With an ungated `kind` (ACT_RELU2) w13 is [E, F, K] and the expert is W2 act(W13 h).
+    `scale_input`: the weight multiplies the expert's INPUT instead of its output, sum_j expert_e(wts[t, j] h_t); the
+    first product being linear, the weight is applied to its fp32 accumulator, act(wts * (W13 h)).
+    Returns fp32 [T, W] (a sum in a fixed order per row)."""
     T, K = h.shape
-    E, F2, _ = w13.shape
-    F_, W, top = F2 // 2, w2.shape[1], ids.shape[1]
+    E = w13.shape[0]
+    gated = kind in (GLU_GELU_TANH, GLU_CLAMPED)
+    F_ = w13.shape[1] // 2 if gated else w13.shape[1]
+    W, top = w2.shape[1], ids.shape[1]
     if not native_device(h):
         out = torch.zeros(T, W)
         hf = h.float()
@@ -686,12 +734,18 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
             tt, jj = torch.nonzero(ids == e, as_tuple=True)
             if tt.numel() == 0:
                 continue
-            gu = (hf[tt] @ w13[e].float().t()).to(h.dtype).float()
-            a = _glu_ref(gu[:, :F_], gu[:, F_:], kind, limit, alpha).to(h.dtype).float()
-            out.index_add_(0, tt, (a @ w2[e].float().t()) * wts[tt, jj][:, None])
+            wt = wts[tt, jj][:, None]
+            gu = hf[tt] @ w13[e].float().t()
+            if scale_input:
+                gu = gu * wt
+            gu = gu.to(h.dtype).float()
+            a = _glu_ref(gu[:, :F_], gu[:, F_:], kind, limit, alpha) if gated else _act_ref(gu, kind)
+            y = a.to(h.dtype).float() @ w2[e].float().t()
+            out.index_add_(0, tt, y if scale_input else y * wt)
         return out
     M = mixers()
     assert h.is_contiguous() and w13.is_contiguous() and w2.is_contiguous() and w13.dtype == w2.dtype == h.dtype
+    assert wts.dtype == torch.float32 and wts.is_contiguous()
     pairs = T * top
     # rows of an expert are padded to whole tiles: 128 / 64-row tiles once the average expert has that many, else 16
     tm = next((t for t in MOE_TILES_BIG if pairs >= t * E), MOE_TILE_SMALL)
@@ -702,12 +756,14 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
     M.moe_align(_i32(ids).data_ptr(), pairs, E, cap, tm, rows.data_ptr(), tile_e.data_ptr(), dest.data_ptr(), stream_ptr())
     act = torch.empty(cap, F_, dtype=h.dtype, device=dev)
     M.grouped_gemm(h.data_ptr(), is_f32(h), h.stride(0), w13.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, tm, top,
-                   F_, K, True, act.data_ptr(), int(kind), float(limit), float(alpha), MOE_MFMA, stream_ptr())
+                   F_, K, 1 if gated else 2, act.data_ptr(), int(kind), float(limit), float(alpha),
+                   wts.data_ptr() if scale_input else 0, MOE_MFMA, stream_ptr())
     y = torch.empty(cap, W, dtype=torch.float32, device=dev)
     M.grouped_gemm(act.data_ptr(), is_f32(act), F_, w2.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, tm, top, W, F_,
-                   False, y.data_ptr(), 0, 0.0, 0.0, MOE_MFMA, stream_ptr())
+                   0, y.data_ptr(), 0, 0.0, 0.0, 0, MOE_MFMA, stream_ptr())
     out = torch.empty(T, W, dtype=torch.float32, device=dev)
-    M.moe_combine(y.data_ptr(), dest.data_ptr(), wts.data_ptr(), T, top, W, out.data_ptr(), stream_ptr())
+    M.moe_combine(y.data_ptr(), dest.data_ptr(), 0 if scale_input else wts.data_ptr(), T, top, W, out.data_ptr(),
+                  stream_ptr())
     return out
 
 
@@ -758,40 +814,56 @@ def post_norm_residual(x: torch.Tensor, y: Optional[torch.Tensor], y_bias: Optio
 # ---------------------------------------------------------------------------- per-head q / k norm, rotation, cache append
 def head_norm_rope_cache(src: torch.Tensor, H: int, G: int, dk: int, dv: int, wq: Optional[torch.Tensor],
                          wk: Optional[torch.Tensor], eps: float, rot: Optional[torch.Tensor], rot_dims: int, sm: SeqMeta,
-                         kcache: torch.Tensor, vcache: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+                         kcache: torch.Tensor, vcache: torch.Tensor, out_dtype: torch.dtype, whole: bool = False,
+                         half: bool = False, v_first: Optional[torch.Tensor] = None,
+                         v_mix: Optional[torch.Tensor] = None) -> torch.Tensor:
     """From rows [q (H dk) | k (G dk) | v (G dv)] (fp32 or an activation tensor, row-strided): every q head and
     every k head is RMS-normed over its own dk entries with one weight of size dk shared by the heads (wq / wk, None
-    = no norm), then the first rot_dims entries of each head are rotated pairwise (entry 2i with 2i + 1) by the
-    table row of the token's position (rot fp32 [positions, rot_dims / 2, 2], None = no rotation). q is returned
-    [T, H dk]; k and v go to cache rows slot_mapping[t]."""
+    = no norm) -- or, with `whole`, q and k are each normed over ALL their entries at once with weights of size H dk /
+    G dk -- then the first rot_dims entries of each head are rotated pairwise (entry 2i with 2i + 1, or, with `half`,
+    entry i with i + rot_dims / 2) by the table row of the token's position (rot fp32 [positions, rot_dims / 2, 2],
+    None = no rotation). With `v_first` ([T, G dv], row-strided, the values another layer projected for the same
+    tokens) and `v_mix` (fp32, one element, lambda) the values become (1 - lambda) v + lambda v_first. q is returned
+    [T, H dk]; k and the (mixed) v go to cache rows slot_mapping[t]."""
     T = src.shape[0]
     nq, nk, nv = H * dk, G * dk, G * dv
     q = torch.empty(T, nq, dtype=out_dtype, device=src.device)
+    assert (v_first is None) == (v_mix is None)
     if native_device(src):
         assert src.stride(1) == 1 and kcache.is_contiguous() and vcache.is_contiguous()
         assert kcache.dtype == vcache.dtype == out_dtype and kcache.shape[-1] == nk and vcache.shape[-1] == nv
         assert rot is None or (rot.dtype == torch.float32 and rot.is_contiguous() and rot.shape[1] * 2 == rot_dims)
         assert rot_dims % 2 == 0 and rot_dims <= dk
+        assert not whole or ((wq is None or wq.numel() == nq) and (wk is None or wk.numel() == nk))
+        if v_first is not None:
+            assert v_first.stride(1) == 1 and v_first.shape == (T, nv) and v_first.dtype == src.dtype
+            assert v_mix.dtype == torch.float32 and v_mix.numel() == 1
         mixers().head_norm_rope_cache(src.data_ptr(), is_f32(src), src.stride(0), H, G, dk, dv, _p(wq), _p(wk),
                                       float(eps), _p(rot), rot.shape[0] if rot is not None else 0,
                                       rot_dims if rot is not None else 0, _i32(sm.positions).data_ptr(),
                                       _i32(sm.slot_mapping).data_ptr(), q.data_ptr(), kcache.data_ptr(),
-                                      vcache.data_ptr(), is_f32(q), T, stream_ptr())
+                                      vcache.data_ptr(), is_f32(q), T, bool(whole), bool(half), _p(v_first),
+                                      v_first.stride(0) if v_first is not None else 0, _p(v_mix), stream_ptr())
         return q
     pf = src.float()
 
     def prep(v, n, w):
+        if w is not None and whole:
+            v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w
         v = v.reshape(T, n, dk)
-        if w is not None:
+        if w is not None and not whole:
             v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w
         if rot is not None and rot_dims:
-            v = _rotate_pairs(v, rot, sm.positions, rot_dims)
+            v = _rotate_pairs(v, rot, sm.positions, rot_dims, half)
         return v.reshape(T, n * dk)
     q.copy_(prep(pf[:, :nq], H, wq).to(out_dtype))
     ok = sm.slot_mapping >= 0
     rows = sm.slot_mapping[ok].long()
     kcache.view(-1, nk)[rows] = prep(pf[:, nq:nq + nk], G, wk)[ok].to(kcache.dtype)
-    vcache.view(-1, nv)[rows] = pf[:, nq + nk:nq + nk + nv][ok].to(vcache.dtype)
+    vals = pf[:, nq + nk:nq + nk + nv]
+    if v_first is not None:
+        vals = (1.0 - v_mix) * vals + v_mix * v_first.float()
+    vcache.view(-1, nv)[rows] = vals[ok].to(vcache.dtype)
     return q
 
 
@@ -937,3 +1009,59 @@ def relu2(z: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     out = torch.empty_like(z)
     mixers().relu2(z.data_ptr(), is_f32(z), _p(bias), out.data_ptr(), z.numel(), z.shape[-1], stream_ptr())
     return out
+
+
+# ---------------------------------------------------------------------------- minimal gated recurrence
+def mingru_scan(proj: torch.Tensor, off_z: int, off_x: int, off_g: int, n: int, bias_z: Optional[torch.Tensor],
+                bias_x: Optional[torch.Tensor], state: torch.Tensor, sm: SeqMeta, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per channel, with z = sigmoid(proj[off_z + c] + bias_z[c]) and u = proj[off_x + c] + bias_x[c]:
+        S <- (1 - z) S + z * cand(u),   cand(u) = u + 1/2 (u >= 0), sigmoid(u) (u < 0)
+    (both gate and candidate read only the current token), and the output S * silu(proj[off_g + c]). proj [T, >= ...]
+    is a row-strided activation tensor; state fp32 [slots, n] is carried and updated. Returns [T, n] as out_dtype."""
+    T = proj.shape[0]
+    out = torch.empty(T, n, dtype=out_dtype, device=proj.device)
+    if native_device(proj):
+        assert proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == n
+        assert max(off_z, off_x, off_g) + n <= proj.shape[1]
+        mixers().mingru_scan(proj.data_ptr(), is_f32(proj), proj.stride(0), off_z, off_x, off_g, n, _p(bias_z), _p(bias_x),
+                             state.data_ptr(), _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
+                             _i32(sm.slots).data_ptr(), out.data_ptr(), is_f32(out), sm.num_seqs, sm.max_q, stream_ptr())
+        return out
+    pf = proj.float()
+    z = torch.sigmoid(pf[:, off_z:off_z + n] + (bias_z if bias_z is not None else 0.0))
+    u = pf[:, off_x:off_x + n] + (bias_x if bias_x is not None else 0.0)
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = pf[:, off_g:off_g + n]
+    g = g * torch.sigmoid(g)
+    qsl, sl, slots = sm.qsl.tolist(), sm.seq_lens.tolist(), sm.slots.tolist()
+    for s in range(sm.num_seqs):
+        lo, hi = qsl[s], qsl[s + 1]
+        if slots[s] < 0 or hi <= lo:
+            out[lo:hi] = 0
+            continue
+        S = state[slots[s]].clone() if sl[s] - (hi - lo) > 0 else torch.zeros(n)
+        for t in range(lo, hi):
+            S = (1.0 - z[t]) * S + z[t] * cand[t]
+            out[t] = (S * g[t]).to(out_dtype)
+        state[slots[s]] = S
+    return out
+
+
+# ---------------------------------------------------------------------------- per-channel decay of a linear recurrence
+def decay_gates(proj: torch.Tensor, off_q: int, off_k: int, n: int, q_scale: float, z: torch.Tensor,
+                z_bias: Optional[torch.Tensor], tau: float):
+    """Inputs of gated_linear_scan with a decay per key channel: q = proj[off_q : off_q + n] * q_scale,
+    k = proj[off_k : off_k + n] and f = sigmoid(z + z_bias)^(1 / tau), evaluated as exp(-softplus(-(z + z_bias)) / tau).
+    proj / z row-strided activation tensors. Returns (q, f, k), fp32 [T, n] each."""
+    T = proj.shape[0]
+    if not native_device(proj):
+        pf = proj.float()
+        zz = z.float() + (z_bias if z_bias is not None else 0.0)
+        f = torch.exp(-torch.nn.functional.softplus(-zz) / tau)
+        return pf[:, off_q:off_q + n] * q_scale, f, pf[:, off_k:off_k + n].clone()
+    assert proj.stride(1) == 1 and z.stride(1) == 1 and z.dtype == proj.dtype and z.shape == (T, n)
+    out = torch.empty(3, T, n, dtype=torch.float32, device=proj.device)
+    mixers().decay_gates(proj.data_ptr(), is_f32(proj), proj.stride(0), off_q, off_k, n, float(q_scale), z.data_ptr(),
+                         z.stride(0), _p(z_bias), float(1.0 / tau), out[0].data_ptr(), out[1].data_ptr(),
+                         out[2].data_ptr(), T, stream_ptr())
+    return out[0], out[1], out[2]
