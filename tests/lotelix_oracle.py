@@ -24,10 +24,6 @@ def group_norm(x, w, groups, eps):
     return unit_rms(x.reshape(T, groups, W // groups), eps).reshape(T, W) * w
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def frequencies(rot):
     n = int(rot["dims"])
     f = torch.tensor([float(rot["base"]) ** (-2.0 * i / n) for i in range(n // 2)], dtype=F64)
@@ -174,13 +170,6 @@ def moe(h, w, pre, mlp):
     return out
 
 
-def router_margin(h, w, pre, mlp):
-    """Smallest gap between the last chosen and the first rejected score over the tokens (how close a call was)."""
-    top = int(mlp["router"]["top"])
-    s = torch.sigmoid(h @ d(w[pre + "router"]).T).sort(-1, descending=True).values
-    return float((s[:, top - 1] - s[:, top]).min()) if s.shape[1] > top else 1.0
-
-
 def forward(cfg, w, tokens, keep=None):
     """Logits [T, vocab] of one whole sequence; `keep` collects the residual stream after every layer."""
     eps, groups = float(cfg["norm"]["eps"]), int(cfg["norm"]["groups"])
@@ -204,3 +193,88 @@ def forward(cfg, w, tokens, keep=None):
         if keep is not None:
             keep.append(x.clone())
     return group_norm(x, d(w["final.norm"]), groups, eps) @ d(w["head"]).T
+
+
+def random_weights(cfg, seed=0):
+    """Random weights of a configuration, rounded to bfloat16 (what a checkpoint stores). `decay_rank` of a right
+    branch (the rank of its decay projection) is read from the mixer's dictionary and not written to config.json."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = cfg["width"], cfg["vocab"]
+    out = {}
+
+    def mat(name, o, i, gain=1.0):
+        out[name] = torch.randn(o, i, generator=g) * gain / math.sqrt(i)
+
+    def vec(name, n, std, mean=0.0):
+        out[name] = torch.randn(n, generator=g) * std + mean
+    out["embed"] = torch.randn(V, W, generator=g) * 0.5
+    mat("head", V, W)
+    vec("final.norm", W, 0.2, 1.0)
+    for n, L in enumerate(cfg["layers"]):
+        pre, m = f"l{n}.", L["mixer"]
+        vec(pre + "norm1", W, 0.2, 1.0)
+        if L["type"] == "mingru":
+            C = m["width"]
+            for nm in ("z", "x", "g"):
+                mat(pre + "mix." + nm, C, W, 2.0)
+            vec(pre + "mix.z.b", C, 0.7)
+            vec(pre + "mix.x.b", C, 0.5)
+            mat(pre + "mix.o", W, C)
+        elif L["type"] == "attention":
+            H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            for nm, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv), ("g", H * dv)):
+                mat(pre + "mix." + nm, rows, W, 2.0)
+            vec(pre + "mix.sink", H, 1.0, 0.5)
+            if m.get("v_mix"):
+                out[pre + "mix.vmix"] = torch.rand((), generator=g) * 0.6 + 0.2
+            mat(pre + "mix.o", W, H * dv)
+        else:
+            a, r = m["left"], m["right"]
+            H, G, dk, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            for nm, rows in (("q", H * dk), ("k", G * dk), ("v", G * dv)):
+                mat(pre + "mix.left." + nm, rows, W, 2.0)
+                vec(pre + "mix.left." + nm + ".b", rows, 0.3)
+            vec(pre + "mix.left.q.norm", H * dk, 0.3, 1.5)
+            vec(pre + "mix.left.k.norm", G * dk, 0.3, 1.5)
+            vec(pre + "mix.left.pb", H, 0.7, -1.5)
+            mat(pre + "mix.left.o", W, H * dv)
+            vec(pre + "mix.left.o.b", W, 0.2)
+            nk, nv, rk = r["heads"] * r["dim"], r["heads"] * r["vdim"], r.get("decay_rank", 4)
+            mat(pre + "mix.right.q", nk, W, 2.0)
+            mat(pre + "mix.right.k", nk, W, 2.0)
+            mat(pre + "mix.right.v", nv, W, 2.0)
+            mat(pre + "mix.right.g", nv, W, 2.0)
+            mat(pre + "mix.right.a1", rk, W, 2.0)
+            mat(pre + "mix.right.a2", nk, rk, 2.0)
+            vec(pre + "mix.right.a2.b", nk, 1.0, 1.5)
+            vec(pre + "mix.right.norm", r["vdim"], 0.3, 1.0)
+            mat(pre + "mix.right.o", W, nv)
+            vec(pre + "mix.left.out", W, 0.3, 1.0)
+            vec(pre + "mix.right.out", W, 0.3, 1.0)
+        mlp = L.get("mlp")
+        if mlp is None:
+            continue
+        vec(pre + "norm2", W, 0.2, 1.0)
+        E, ff = mlp["router"]["experts"], mlp["expert"]["ff"]
+        mat(pre + "mlp.router", E, W, 4.0)
+        for e in range(E):
+            mat(f"{pre}mlp.e{e}.up", ff, W, 1.5)
+            mat(f"{pre}mlp.e{e}.down", W, ff)
+    return {k: v.to(torch.bfloat16).to(F64) for k, v in out.items()}
+
+
+def write_checkpoint(path, cfg, Wt):
+    """config.json + model.safetensors (bfloat16) of a test model."""
+    import copy
+    import json
+    import os
+
+    from safetensors.torch import save_file
+    c = copy.deepcopy(cfg)
+    for L in c["layers"]:
+        if L["type"] == "parallel":
+            L["mixer"]["right"].pop("decay_rank", None)
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(c, f)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in Wt.items()}, os.path.join(path, "model.safetensors"))
