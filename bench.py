@@ -85,6 +85,12 @@ def parse():
                          "--dofivik-prompts, --dofivik-context apply)")
     ap.add_argument("--loluzen-sizes", default="1b-class,8b-class")
     ap.add_argument("--loluzen-only", default=None, choices=["loluzen", "llama"])
+    ap.add_argument("--lotelix", action="store_true",
+                    help="instead of the headline: prefill and decode tokens/s of Lotelix beside a Mixtral-type model "
+                         "and a Llama of equal layer sizes (bench/lotelix_bench.py; --prompt-len, --concurrency = decode "
+                         "batch, --steps, --warmup, --dofivik-prompts, --dofivik-context apply)")
+    ap.add_argument("--lotelix-sizes", default="1b-class,8b-class")
+    ap.add_argument("--lotelix-only", default=None, choices=["lotelix", "mixtral", "llama"])
     return ap.parse_args()
 
 
@@ -179,11 +185,12 @@ def preflight(st, world: int, tp: int, dev, eng) -> dict:
 
 def main():
     a = parse()
-    if a.dofivik or a.vizonex or a.loluzen:
+    if a.dofivik or a.vizonex or a.loluzen or a.lotelix:
         import importlib.util
         here = os.path.dirname(os.path.abspath(__file__))
         sys.path.insert(0, here)
-        which = "dofivik_bench" if a.dofivik else "vizonex_bench" if a.vizonex else "loluzen_bench"
+        which = "dofivik_bench" if a.dofivik else "vizonex_bench" if a.vizonex else "loluzen_bench" if a.loluzen \
+            else "lotelix_bench"
         spec = importlib.util.spec_from_file_location(which, os.path.join(here, "bench", which + ".py"))
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)

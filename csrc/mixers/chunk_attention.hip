@@ -212,7 +212,15 @@ __device__ __forceinline__ float exp2_fast(float x) {
 #endif
 }
 
-template <int NKK_MAX, int NMT_MAX, int NW>
+__device__ __forceinline__ float rcp_fast(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_rcpf(x);
+#else
+  return 1.f / x;
+#endif
+}
+
+template <int NKK_MAX, int NMT_MAX, int NW, int WFN>
 __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int32_t* __restrict__ block_tables, int bt_width, int bs, const int32_t* __restrict__ qsl,
@@ -220,7 +228,7 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
     const float* __restrict__ sink, bf16* __restrict__ out, int H, int G, int dk, int dv_head, int mask, int size,
     float scale, int RH, int head_slots, float* __restrict__ part_o, float* __restrict__ part_ml, int Ttot,
     const bf16* __restrict__ gate, int64_t ld_gate, const float* __restrict__ r1, const float* __restrict__ r2, int vmode,
-    int gate_elem, int wfn, const float* __restrict__ hbias) {
+    int gate_elem, const float* __restrict__ hbias) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   // dv: value columns per query head; voff: where they start in a cached row of G * dv_head values
   const int dv = vmode == kValuesAll ? G * dv_head : dv_head;
@@ -289,7 +297,7 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
   // the sink starts the running softmax: weight exp(sink - m) = 1 with no value behind it
   const bool with_sink = sink && (nsplit == 1 || blockIdx.x == 0);  // the sink enters the first share only
   float m = with_sink ? sink[head] * kLog2e : -INFINITY, l = with_sink ? 1.f : 0.f;
-  const bool sig = wfn == kWeightsSigmoid;
+  constexpr bool sig = WFN == kWeightsSigmoid;
   const float sbias = (sig && hbias) ? hbias[head] * kLog2e : 0.f;   // the per-head score bias, in units of ln 2
 
   // staging: thread -> (row = tid / NW, 16-byte chunks tid % NW, + NW, ..) of the K row and of the V row. The next
@@ -357,12 +365,12 @@ __global__ __launch_bounds__(64 * NW) void masked_attention_mfma_kernel(
         sacc[n][r] = v;
         mx = fmaxf(mx, v);
       }
-    if (sig) {
+    if constexpr (sig) {
       // weight = sigmoid(score + bias) = 1 / (1 + 2^-(s + b)) with s, b in units of ln 2; an unseen key (-inf) weighs 0
 #pragma unroll
       for (int n = 0; n < 4; ++n)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sacc[n][r] = __frcp_rn(1.f + exp2_fast(-(sacc[n][r] + sbias)));
+        for (int r = 0; r < 4; ++r) sacc[n][r] = rcp_fast(1.f + exp2_fast(-(sacc[n][r] + sbias)));
     } else {
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -782,11 +790,17 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
   if (!head_slots || nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) nsplit = 1;
   if (head_slots) grid = dim3(nsplit, G, ns);
   const size_t lds = (size_t)kKT * (dk + 8 + dv + 8) * sizeof(uint16_t);
-#define XGM_MK(NKK, NMT, NW)                                                                                          \
-  masked_attention_mfma_kernel<NKK, NMT, NW><<<grid, 64 * NW, lds, st>>>(                                             \
+#define XGM_MK2(NKK, NMT, NW, WFN)                                                                                    \
+  masked_attention_mfma_kernel<NKK, NMT, NW, WFN><<<grid, 64 * NW, lds, st>>>(                                        \
       (const bf16*)q, (const bf16*)kcache, (const bf16*)vcache, block_tables, bt_width, bs, qsl, seq_lens, slots, temp, \
       sink, (bf16*)out, H, G, dk, dv_head, mask, size, scale, RH, head_slots, part_o, part_ml, T_, (const bf16*)gate,  \
-      ld_gate, r1, r2, vmode, ge, wfn, hbias);
+      ld_gate, r1, r2, vmode, ge, hbias);
+#define XGM_MK(NKK, NMT, NW)                  \
+  if (wfn == kWeightsSigmoid) {               \
+    XGM_MK2(NKK, NMT, NW, kWeightsSigmoid)    \
+  } else {                                    \
+    XGM_MK2(NKK, NMT, NW, kWeightsSoftmax)    \
+  }
 #define XGM_MM(NKK, NMT)                                                                                              \
   if (nw == 16 && NMT <= 8) {                                                                                         \
     XGM_MK(NKK, NMT, (NMT <= 8 ? 16 : 8))                                                                             \
@@ -805,6 +819,7 @@ int masked_attention_mfma(const void* q, const void* kcache, const void* vcache,
   return -2;
 #undef XGM_MM
 #undef XGM_MK
+#undef XGM_MK2
 }
 
 void talk_mix(const void* o_all, bool f32, const float* talk, const void* gate, int64_t ld_gate, void* out, int T_, int H,

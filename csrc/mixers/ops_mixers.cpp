@@ -15,7 +15,8 @@ void embed_rows(const int32_t*, const void*, bool, float*, int, int, int, const 
 void causal_conv(const void*, bool, int64_t, const float*, const float*, float*, const int32_t*, const int32_t*,
                  const int32_t*, void*, bool, int, int, int, int, bool, bool, hipStream_t);
 int residual_norm(float*, const void*, int64_t, const float*, const void*, int64_t, const float*, const float*, bool,
-                  const float*, float, float*, void*, bool, int, int, int, const float*, const float*, hipStream_t);
+                  const float*, float, float*, void*, bool, int, int, int, const float*, const float*, const int32_t*,
+                  const float*, int, hipStream_t);
 void qk_norm_cache(const void*, bool, int64_t, int, int, int, const float*, const float*, float, const int32_t*, void*,
                    void*, void*, int, hipStream_t);
 int masked_attention(const void*, bool, const void*, const void*, const int32_t*, int, int, const int32_t*,
@@ -45,12 +46,14 @@ int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, con
 void gated_group_norm(const float*, const void*, bool, int64_t, const float*, int, float, void*, int, int, int, bool,
                       hipStream_t);
 void glu_act(const void*, bool, int64_t, void*, int, int, int, float, float, hipStream_t);
-int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, hipStream_t);
+int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, const float*,
+                   const float*, int, hipStream_t);
 int moe_align(const int32_t*, int, int, int, int, int32_t*, int32_t*, int32_t*, hipStream_t);
 int grouped_gemm(const void*, bool, int64_t, const void*, const int32_t*, const int32_t*, int, int, int, int, int, int, void*,
                  int, float, float, const float*, bool, hipStream_t);
 int mingru_scan(const void*, bool, int64_t, int, int, int, int, const float*, const float*, float*, const int32_t*,
-                const int32_t*, const int32_t*, void*, bool, int, int, hipStream_t);
+                const int32_t*, const int32_t*, void*, bool, int, int, float*, int, hipStream_t);
+int64_t mingru_scratch_floats(int, int, int);
 void decay_gates(const void*, bool, int64_t, int, int, int, float, const void*, int64_t, const float*, float, float*, float*,
                  float*, int, hipStream_t);
 void moe_combine(const float*, const int32_t*, const float*, int, int, int, float*, hipStream_t);
@@ -103,11 +106,13 @@ PYBIND11_MODULE(_mixers, m) {
   });
   m.def("residual_norm", [](uintptr_t x, uintptr_t y1, int64_t ld1, uintptr_t a1, uintptr_t y2, int64_t ld2, uintptr_t y3,
                             uintptr_t a2, bool y_f32, uintptr_t g, float eps, uintptr_t n32, uintptr_t nact,
-                            bool nact_f32, int T, int W, int groups, uintptr_t bw1, uintptr_t bw2, uintptr_t st) {
+                            bool nact_f32, int T, int W, int groups, uintptr_t bw1, uintptr_t bw2, uintptr_t dest,
+                            uintptr_t cw, int top, uintptr_t st) {
     if ((y1 && ld1 < W) || (y2 && ld2 < W)) throw std::invalid_argument("residual_norm: row stride smaller than the width");
     int rc = xgm::residual_norm(P<float>(x), P<const void>(y1), ld1, P<const float>(a1), P<const void>(y2), ld2,
                                 P<const float>(y3), P<const float>(a2), y_f32, P<const float>(g), eps, P<float>(n32),
-                                P<void>(nact), nact_f32, T, W, groups, P<const float>(bw1), P<const float>(bw2), S(st));
+                                P<void>(nact), nact_f32, T, W, groups, P<const float>(bw1), P<const float>(bw2),
+                                P<const int32_t>(dest), P<const float>(cw), top, S(st));
     check(rc, "residual_norm");
   });
   m.def("qk_norm_cache", [](uintptr_t proj, bool f32, int64_t ld, int nq, int nk, int nv, uintptr_t wq, uintptr_t wk,
@@ -247,9 +252,11 @@ PYBIND11_MODULE(_mixers, m) {
     check(0, "glu_act");
   });
   m.def("grouped_router", [](uintptr_t logits, uintptr_t corr, int T, int E, int count, int keep, int top, float scale,
-                             uintptr_t ids, uintptr_t wts, uintptr_t st) {
+                             uintptr_t ids, uintptr_t wts, uintptr_t x, uintptr_t rw, int W, uintptr_t st) {
+    if ((x != 0) != (rw != 0) || (x && W < 1) || (!x && !logits))
+      throw std::invalid_argument("grouped_router: needs logits, or rows and router weights");
     int rc = xgm::grouped_router(P<const float>(logits), P<const float>(corr), T, E, count, keep, top, scale,
-                                 P<int32_t>(ids), P<float>(wts), S(st));
+                                 P<int32_t>(ids), P<float>(wts), P<const float>(x), P<const float>(rw), W, S(st));
     check(rc, "grouped_router");
   });
   m.def("moe_align", [](uintptr_t ids, int pairs, int E, int cap, int tm, uintptr_t rows, uintptr_t tile_expert,
@@ -274,14 +281,15 @@ PYBIND11_MODULE(_mixers, m) {
 
   m.def("mingru_scan", [](uintptr_t proj, bool f32, int64_t ld, int off_z, int off_x, int off_g, int n, uintptr_t bz,
                           uintptr_t bx, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t out,
-                          bool out_f32, int ns, int max_q, uintptr_t st) {
+                          bool out_f32, int ns, int max_q, uintptr_t scratch, int T, uintptr_t st) {
     if (n < 1 || off_z < 0 || off_x < 0 || off_g < 0 || ld < off_z + n || ld < off_x + n || ld < off_g + n || !state)
       throw std::invalid_argument("mingru_scan: columns outside the row");
     int rc = xgm::mingru_scan(P<const void>(proj), f32, ld, off_z, off_x, off_g, n, P<const float>(bz), P<const float>(bx),
                               P<float>(state), P<const int32_t>(qsl), P<const int32_t>(sl), P<const int32_t>(slots),
-                              P<void>(out), out_f32, ns, max_q, S(st));
+                              P<void>(out), out_f32, ns, max_q, P<float>(scratch), T, S(st));
     check(rc, "mingru_scan");
   });
+  m.def("mingru_scratch_floats", [](int T, int ns, int n) { return xgm::mingru_scratch_floats(T, ns, n); });
   m.def("decay_gates", [](uintptr_t proj, bool f32, int64_t ld, int off_q, int off_k, int n, float q_scale, uintptr_t z,
                           int64_t ld_z, uintptr_t zb, float inv_tau, uintptr_t q, uintptr_t f, uintptr_t k, int T,
                           uintptr_t st) {

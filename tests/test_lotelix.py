@@ -447,10 +447,14 @@ def test_rotation_frequencies_in_all_three_ranges():
 
 @pytest.mark.parametrize("device", OP_CASES)
 @pytest.mark.parametrize("n,cuts", [(70, [[1, 1, 1, 3, 16, 1, 17, 40, 1, 128, 129, 2, 300], [2, 5, 1, 1, 1, 1, 200, 7, 1, 1, 1, 1, 1]]),
-                                    (64, [[400], [1] * 6]), (200, [[17, 130], [131, 16]])])
-def test_minimal_gated_recurrence_over_portions_and_slots(device, n, cuts):
-    """Steps of single tokens, short and long portions (every workgroup shape of the scan), two sequences sharing
-    steps, a slot with another sequence's leftovers, columns of a wider strided row."""
+                                    (64, [[400], [1] * 6]), (200, [[17, 130], [131, 16]]),
+                                    (130, [[3, 1300, 1, 257], [700, 2, 513, 1]]), (64, [[900, 1, 600], [5, 1, 1]])])
+@pytest.mark.parametrize("two_pass", [True, False], ids=["chunks", "one-workgroup"])
+def test_minimal_gated_recurrence_over_portions_and_slots(device, n, cuts, two_pass, monkeypatch):
+    """Steps of single tokens, short and long portions (every workgroup shape of the scan; the longest ones as chunks
+    over the whole grid, in two launches), two sequences sharing steps, a slot with another sequence's leftovers,
+    columns of a wider strided row."""
+    monkeypatch.setattr(sq, "MINGRU_TWO_PASS", two_pass)
     g = torch.Generator().manual_seed(n)
     W = 24
     cfg = {"width": W, "vocab": 8, "layers": [{"type": "mingru", "mixer": {"width": n}, "mlp": None}]}
@@ -668,6 +672,24 @@ def test_experts_scaled_at_their_input(device, dtype, T, E, top, K, F_):
     down = torch.stack([w[f"e{e}.down"] for e in range(E)]).to(dt).to(device)
     got = sq.routed_experts(h.to(dt).to(device), up, down, ids, wts, sq.ACT_RELU2, scale_input=True)
     assert rel_err(got, ref) < (1e-4 if dtype == "float32" else 3e-2)
+    # the logits formed inside the router kernel; the sum over a token's choices inside the residual update
+    ids2, wts2 = sq.grouped_router(None, None, 1, 1, top, 1.0, rows=h.float().to(device),
+                                   router_w=w["router"].float().to(device))
+    assert torch.equal(ids2.cpu().long().sort(-1).values, ids.cpu().long().sort(-1).values)
+    assert float((wts2.sort(-1).values - wts.sort(-1).values).abs().max()) < 1e-5
+    rows = sq.routed_experts(h.to(dt).to(device), up, down, ids, wts, sq.ACT_RELU2, scale_input=True, combine=False)
+    x = torch.randn(T, K, generator=g)
+    xs = x.clone().to(device)
+    nw = (torch.rand(K, generator=g) + 0.5)
+    _, n = sq.residual_norm(xs, None, None, None, rows, None, nw.to(device), 1e-5, torch.float32, False, 2)
+    assert rel_err(xs, x.to(F64) + ref) < (1e-4 if dtype == "float32" else 3e-2)
+    assert rel_err(n, orc.group_norm(x.to(F64) + ref, nw.to(F64), 2, 1e-5)) < (1e-4 if dtype == "float32" else 3e-2)
+    # weights applied at the output: the same rows with a weight per choice
+    plain = sq.routed_experts(h.to(dt).to(device), up, down, ids, wts, sq.ACT_RELU2)
+    rows = sq.routed_experts(h.to(dt).to(device), up, down, ids, wts, sq.ACT_RELU2, combine=False)
+    xs = torch.zeros(T, K, device=device)
+    sq.residual_norm(xs, None, None, None, rows, None, None, 1e-5)
+    assert rel_err(xs, plain.cpu().to(F64)) < 1e-5
 
 
 # ---------------------------------------------------------------------------------- random configurations

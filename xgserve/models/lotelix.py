@@ -175,9 +175,9 @@ class InputScaledMoE(nn.Module):
         self.down = _p(torch.empty(self.E, width, self.ff, device=device, dtype=dtype))
 
     def forward(self, n32, nact):
-        """The routed sum, fp32 [T, W]."""
-        ids, wts = sq.grouped_router(F.linear(n32, self.router), None, 1, 1, self.top, 1.0)
-        return sq.routed_experts(nact, self.up, self.down, ids, wts, sq.ACT_RELU2, scale_input=True)
+        """The experts' output rows; the residual update sums them per token."""
+        ids, wts = sq.grouped_router(None, None, 1, 1, self.top, 1.0, rows=n32, router_w=self.router)
+        return sq.routed_experts(nact, self.up, self.down, ids, wts, sq.ACT_RELU2, scale_input=True, combine=False)
 
 
 class LotelixLayer(nn.Module):

@@ -407,14 +407,24 @@ def residual_norm(x: torch.Tensor, y1: Optional[torch.Tensor], a1: Optional[torc
     """x <- x + a1 * y1 + a2 * (y2 + y3) in place (x fp32 [T, W]; y1 / y2 activation tensors, y3 fp32; a1 / a2
     per-channel scales, None = 1; any y may be None), then, with `norm_w`, the RMS norm of the new x:
     n = x / sqrt(mean(x^2) + eps) * norm_w, returned as (n fp32 or None, n as out_dtype or None).
+    y3 may be the `RoutedRows` of routed_experts(combine=False): the weighted sum over a token's choices is then formed here.
     `groups` > 1: the norm splits a row into that many equal consecutive parts, each divided by its own root mean
     square. `branch_w` = (w1, w2): y1 and y2 are the outputs of two branches that are averaged after each is
     RMS-normed over the row with its plain weight, x <- x + (N0(y1) w1 + N0(y2) w2) / 2 + y3 (no a1 / a2)."""
     T, W = x.shape
     assert groups >= 1 and W % groups == 0
+    routed = None
+    if isinstance(y3, RoutedRows):   # the rows of a routed mixture, summed per token here
+        if y3.dest is None:
+            y3 = y3.y
+        else:
+            routed, y3 = y3, y3.y
     if not native_device(x):
         def n0(v):
             return v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        if routed is not None:
+            rows = y3[routed.dest.long()]                         # [T, top, W]
+            y3 = (rows * routed.wts[:, :, None]).sum(1) if routed.wts is not None else rows.sum(1)
         v = x
         if branch_w is not None:
             v = v + 0.5 * (n0(y1.float()) * branch_w[0] + n0(y2.float()) * branch_w[1])
@@ -435,14 +445,18 @@ def residual_norm(x: torch.Tensor, y1: Optional[torch.Tensor], a1: Optional[torc
     assert x.dtype == torch.float32 and x.is_contiguous()
     ys = [y for y in (y1, y2) if y is not None]
     assert all(y.stride(1) == 1 and y.shape == x.shape for y in ys) and len({y.dtype for y in ys}) <= 1
-    assert y3 is None or (y3.dtype == torch.float32 and y3.is_contiguous() and y3.shape == x.shape)
+    assert y3 is None or (y3.dtype == torch.float32 and y3.is_contiguous() and (routed is not None or y3.shape == x.shape))
+    if routed is not None:
+        assert y3.shape[1] == W and routed.dest.dtype == torch.int32 and routed.dest.is_contiguous()
+        assert routed.dest.shape[0] == T and (routed.wts is None or routed.wts.shape == routed.dest.shape)
     n32 = torch.empty_like(x) if (norm_w is not None and want_f32) else None
     nact = torch.empty(T, W, dtype=out_dtype, device=x.device) if (norm_w is not None and out_dtype is not None) else None
     mixers().residual_norm(x.data_ptr(), _p(y1), y1.stride(0) if y1 is not None else 0, _p(a1), _p(y2),
                            y2.stride(0) if y2 is not None else 0, _p(y3), _p(a2), is_f32(ys[0]) if ys else True,
                            _p(norm_w), float(eps), _p(n32), _p(nact), is_f32(nact) if nact is not None else True, T, W,
                            int(groups), _p(branch_w[0]) if branch_w else 0, _p(branch_w[1]) if branch_w else 0,
-                           stream_ptr())
+                           _p(routed.dest) if routed else 0, _p(routed.wts) if routed else 0,
+                           routed.dest.shape[1] if routed else 0, stream_ptr())
     return n32, nact
 
 
@@ -684,15 +698,23 @@ def glu_act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.702
     return out
 
 
-def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], count: int, keep: int, top: int,
-                   scale: float):
-    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]). Scores are
+def grouped_router(logits: Optional[torch.Tensor], correction: Optional[torch.Tensor], count: int, keep: int, top: int,
+                   scale: float, rows: Optional[torch.Tensor] = None, router_w: Optional[torch.Tensor] = None):
+    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]); with `rows` (fp32 [T, W]) and
+    `router_w` (fp32 [E, W]) instead of `logits`, the logits rows . router_w[e] are formed in fp32 inside. Scores are
     sigmoid(logits). Selection uses score + correction: the experts form `count` contiguous groups of equal
     size, a group is rated by the sum of its two highest selection scores, and only members of the `keep`
     highest-rated groups are eligible (everything else is excluded outright, selection score -inf). The
     returned weights are score * scale: the correction does not enter them and they are not normalised."""
-    T, E = logits.shape
-    if not native_device(logits):
+    if logits is None:
+        assert rows.dtype == router_w.dtype == torch.float32 and rows.shape[1] == router_w.shape[1]
+        if not native_device(rows):
+            logits = rows @ router_w.t()
+    if logits is not None:
+        T, E = logits.shape
+    else:
+        T, E = rows.shape[0], router_w.shape[0]
+    if logits is not None and not native_device(logits):
         s = torch.sigmoid(logits.float())
         c = s + (correction if correction is not None else 0.0)
         per = E // count
@@ -702,11 +724,13 @@ def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], cou
         c = c.masked_fill(~kept.repeat_interleave(per, 1), float("-inf"))
         ids = c.topk(top, -1).indices
         return ids.to(torch.int32), s.gather(1, ids) * scale
-    assert logits.dtype == torch.float32 and logits.is_contiguous()
-    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
-    wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    mixers().grouped_router(logits.data_ptr(), _p(correction), T, E, int(count), int(keep), int(top), float(scale),
-                            ids.data_ptr(), wts.data_ptr(), stream_ptr())
+    src = logits if logits is not None else rows
+    assert src.dtype == torch.float32 and src.is_contiguous() and (logits is not None or router_w.is_contiguous())
+    ids = torch.empty(T, top, dtype=torch.int32, device=src.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=src.device)
+    mixers().grouped_router(_p(logits), _p(correction), T, E, int(count), int(keep), int(top), float(scale),
+                            ids.data_ptr(), wts.data_ptr(), _p(rows) if logits is None else 0,
+                            _p(router_w) if logits is None else 0, rows.shape[1] if logits is None else 0, stream_ptr())
     return ids, wts
 
 
@@ -715,13 +739,23 @@ def _act_ref(z, kind):
     return torch.relu(z).pow(2)
 
 
+@dataclass
+class RoutedRows:
+    """The experts' output rows before they are summed per token (routed_experts(combine=False)): row dest[t, j] of
+    `y` (fp32, the sorted layout) is token t's j-th choice, to be weighted by wts[t, j] (None: 1). residual_norm takes
+    it in place of its fp32 term and forms the sum itself. `dest` None: `y` is the finished sum [T, W]."""
+    y: torch.Tensor
+    dest: Optional[torch.Tensor] = None
+    wts: Optional[torch.Tensor] = None
+
+
 def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, kind: int,
-                   limit: float = 0.0, alpha: float = 1.702, scale_input: bool = False) -> torch.Tensor:
+                   limit: float = 0.0, alpha: float = 1.702, scale_input: bool = False, combine: bool = True):
     """sum_j wts[t, j] * W2[e] glu(W13[e] h_t), e = ids[t, j]. w13 [E, 2 F, K] holds each expert's gate rows then
     its up rows, w2 [E, W, F]. With an ungated `kind` (ACT_RELU2) w13 is [E, F, K] and the expert is W2 act(W13 h).
     `scale_input`: the weight multiplies the expert's INPUT instead of its output, sum_j expert_e(wts[t, j] h_t); the
     first product being linear, the weight is applied to its fp32 accumulator, act(wts * (W13 h)).
-    Returns fp32 [T, W] (a sum in a fixed order per row)."""
+    Returns fp32 [T, W] (a sum in a fixed order per row), or with combine=False the rows as `RoutedRows`."""
     T, K = h.shape
     E = w13.shape[0]
     gated = kind in (GLU_GELU_TANH, GLU_CLAMPED)
@@ -742,7 +776,7 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
             a = _glu_ref(gu[:, :F_], gu[:, F_:], kind, limit, alpha) if gated else _act_ref(gu, kind)
             y = a.to(h.dtype).float() @ w2[e].float().t()
             out.index_add_(0, tt, y if scale_input else y * wt)
-        return out
+        return out if combine else RoutedRows(out)
     M = mixers()
     assert h.is_contiguous() and w13.is_contiguous() and w2.is_contiguous() and w13.dtype == w2.dtype == h.dtype
     assert wts.dtype == torch.float32 and wts.is_contiguous()
@@ -761,6 +795,8 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
     y = torch.empty(cap, W, dtype=torch.float32, device=dev)
     M.grouped_gemm(act.data_ptr(), is_f32(act), F_, w2.data_ptr(), rows.data_ptr(), tile_e.data_ptr(), cap, tm, top, W, F_,
                    0, y.data_ptr(), 0, 0.0, 0.0, 0, MOE_MFMA, stream_ptr())
+    if not combine:
+        return RoutedRows(y, dest.view(T, top), None if scale_input else wts)
     out = torch.empty(T, W, dtype=torch.float32, device=dev)
     M.moe_combine(y.data_ptr(), dest.data_ptr(), 0 if scale_input else wts.data_ptr(), T, top, W, out.data_ptr(),
                   stream_ptr())
@@ -1012,6 +1048,11 @@ def relu2(z: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------- minimal gated recurrence
+# XGS_TUNE mingru_two_pass=0: every portion in one workgroup per (sequence, 64 channels) (A/B and tests)
+MINGRU_TWO_PASS = tune.get_bool("mingru_two_pass", True)
+MINGRU_TWO_PASS_MIN = 512   # portions longer than this are scanned as chunks of 256 tokens over the whole grid
+
+
 def mingru_scan(proj: torch.Tensor, off_z: int, off_x: int, off_g: int, n: int, bias_z: Optional[torch.Tensor],
                 bias_x: Optional[torch.Tensor], state: torch.Tensor, sm: SeqMeta, out_dtype: torch.dtype) -> torch.Tensor:
     """Per channel, with z = sigmoid(proj[off_z + c] + bias_z[c]) and u = proj[off_x + c] + bias_x[c]:
@@ -1023,9 +1064,13 @@ def mingru_scan(proj: torch.Tensor, off_z: int, off_x: int, off_g: int, n: int, 
     if native_device(proj):
         assert proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == n
         assert max(off_z, off_x, off_g) + n <= proj.shape[1]
+        scratch = None
+        if MINGRU_TWO_PASS and sm.max_q > MINGRU_TWO_PASS_MIN:   # a long portion: its pieces spread over the whole grid
+            scratch = torch.empty(mixers().mingru_scratch_floats(T, sm.num_seqs, n), dtype=torch.float32, device=proj.device)
         mixers().mingru_scan(proj.data_ptr(), is_f32(proj), proj.stride(0), off_z, off_x, off_g, n, _p(bias_z), _p(bias_x),
                              state.data_ptr(), _i32(sm.qsl).data_ptr(), _i32(sm.seq_lens).data_ptr(),
-                             _i32(sm.slots).data_ptr(), out.data_ptr(), is_f32(out), sm.num_seqs, sm.max_q, stream_ptr())
+                             _i32(sm.slots).data_ptr(), out.data_ptr(), is_f32(out), sm.num_seqs, sm.max_q, _p(scratch), T,
+                             stream_ptr())
         return out
     pf = proj.float()
     z = torch.sigmoid(pf[:, off_z:off_z + n] + (bias_z if bias_z is not None else 0.0))
