@@ -392,7 +392,7 @@ def in_portions(device, xs, cuts, slots, fn, tables=None, block_size=4):
                 parts.append(xs[i][at[i]:at[i] + q])
                 who.append((i, q))
                 at[i] += q
-        sm = seq_meta(device, rows, block_size, [tables[i] if tables else [0] * 256 for i, _ in who])
+        sm = seq_meta(device, rows, block_size, [tables[i] if tables else [0] * 512 for i, _ in who])
         y = fn(torch.cat(parts).to(device), sm)
         o = 0
         for i, q in who:
