@@ -7,9 +7,7 @@
 //                    split into `count` contiguous groups of equal size, a group is rated by the sum of its two
 //                    highest selection scores, members of the `keep` highest-rated groups stay eligible (all
 //                    others are excluded outright: selection score -inf); the `top` highest eligible selection
-//                    scores win; weight = score * scale (the correction does not enter it, no normalisation).
-//                    With rows x [T][W] and router weights rw [E][W] (both fp32) the logits x . rw[e] are formed
-//                    here, in fp32, instead of being read.
+//                    scores win; weight = score * scale (the correction does not enter it, no normalisation)
 //   moe_align        (token, choice) pairs sorted by expert into tiles of `tm` rows (padded with -1)
 //   grouped_gemm     per tile: rows x expert weights, in one of three modes:
 //                      kGemmRows    A rows as they lie in the sorted layout -> fp32 rows (the second product)
@@ -62,43 +60,20 @@ constexpr int kMaxEPL = 8;  // experts per lane: E <= 512
 
 __global__ __launch_bounds__(64) void grouped_router_kernel(const float* __restrict__ logits, const float* __restrict__ corr,
                                                             int E, int count, int keep, int top, float scale,
-                                                            int32_t* __restrict__ ids, float* __restrict__ wts,
-                                                            const float* __restrict__ x, const float* __restrict__ rw,
-                                                            int W) {
+                                                            int32_t* __restrict__ ids, float* __restrict__ wts) {
   extern __shared__ float sm[];
   float* cs = sm;              // [E] choice scores
   float* gs = sm + E;          // [count] group scores
   int* kept = (int*)(gs + count);  // [count]
-  float* lg = (float*)(kept + count);  // [E] logits formed here (x != nullptr)
   const int t = blockIdx.x, lane = threadIdx.x;
   const int per = E / count;
-  if (x) {  // one dot product per expert, the wave's lanes striding over the row
-    const float* xr = x + (int64_t)t * W;
-    for (int e = 0; e < E; ++e) {
-      const float* wr = rw + (int64_t)e * W;
-      float acc = 0.f;
-      if ((W & 3) == 0) {
-        for (int c = 4 * lane; c < W; c += 256) {
-          float a[4], b[4];
-          ld4(xr + c, a);
-          ld4(wr + c, b);
-          acc += a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
-        }
-      } else {
-        for (int c = lane; c < W; c += 64) acc += xr[c] * wr[c];
-      }
-      acc = wave_sum(acc);
-      if (lane == 0) lg[e] = acc;
-    }
-    __syncthreads();
-  }
   float sc[kMaxEPL], ch[kMaxEPL];
 #pragma unroll
   for (int i = 0; i < kMaxEPL; ++i) {
     const int e = lane + 64 * i;
     sc[i] = 0.f, ch[i] = -INFINITY;
     if (e < E) {
-      sc[i] = sigmoidf(x ? lg[e] : logits[(int64_t)t * E + e]);
+      sc[i] = sigmoidf(logits[(int64_t)t * E + e]);
       ch[i] = sc[i] + (corr ? corr[e] : 0.f);
       cs[e] = ch[i];
     }
@@ -492,13 +467,12 @@ void glu_act(const void* in, bool f32, int64_t ld, void* out, int T_, int F, int
 }
 
 int grouped_router(const float* logits, const float* corr, int T_, int E, int count, int keep, int top, float scale,
-                   int32_t* ids, float* wts, const float* x, const float* rw, int W, hipStream_t st) {
+                   int32_t* ids, float* wts, hipStream_t st) {
   if (T_ <= 0) return 0;
   if (E < 1 || E > 64 * kMaxEPL || count < 1 || E % count != 0 || keep < 1 || keep > count || top < 1 ||
       top > keep * (E / count))
     return -1;
-  grouped_router_kernel<<<T_, 64, (2 * E + 2 * count) * sizeof(float), st>>>(logits, corr, E, count, keep, top, scale, ids,
-                                                                             wts, x, rw, W);
+  grouped_router_kernel<<<T_, 64, (E + 2 * count) * sizeof(float), st>>>(logits, corr, E, count, keep, top, scale, ids, wts);
   return 0;
 }
 

@@ -698,23 +698,15 @@ def glu_act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.702
     return out
 
 
-def grouped_router(logits: Optional[torch.Tensor], correction: Optional[torch.Tensor], count: int, keep: int, top: int,
-                   scale: float, rows: Optional[torch.Tensor] = None, router_w: Optional[torch.Tensor] = None):
-    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]); with `rows` (fp32 [T, W]) and
-    `router_w` (fp32 [E, W]) instead of `logits`, the logits rows . router_w[e] are formed in fp32 inside. Scores are
+def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], count: int, keep: int, top: int,
+                   scale: float):
+    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]). Scores are
     sigmoid(logits). Selection uses score + correction: the experts form `count` contiguous groups of equal
     size, a group is rated by the sum of its two highest selection scores, and only members of the `keep`
     highest-rated groups are eligible (everything else is excluded outright, selection score -inf). The
     returned weights are score * scale: the correction does not enter them and they are not normalised."""
-    if logits is None:
-        assert rows.dtype == router_w.dtype == torch.float32 and rows.shape[1] == router_w.shape[1]
-        if not native_device(rows):
-            logits = rows @ router_w.t()
-    if logits is not None:
-        T, E = logits.shape
-    else:
-        T, E = rows.shape[0], router_w.shape[0]
-    if logits is not None and not native_device(logits):
+    T, E = logits.shape
+    if not native_device(logits):
         s = torch.sigmoid(logits.float())
         c = s + (correction if correction is not None else 0.0)
         per = E // count
@@ -724,13 +716,11 @@ def grouped_router(logits: Optional[torch.Tensor], correction: Optional[torch.Te
         c = c.masked_fill(~kept.repeat_interleave(per, 1), float("-inf"))
         ids = c.topk(top, -1).indices
         return ids.to(torch.int32), s.gather(1, ids) * scale
-    src = logits if logits is not None else rows
-    assert src.dtype == torch.float32 and src.is_contiguous() and (logits is not None or router_w.is_contiguous())
-    ids = torch.empty(T, top, dtype=torch.int32, device=src.device)
-    wts = torch.empty(T, top, dtype=torch.float32, device=src.device)
-    mixers().grouped_router(_p(logits), _p(correction), T, E, int(count), int(keep), int(top), float(scale),
-                            ids.data_ptr(), wts.data_ptr(), _p(rows) if logits is None else 0,
-                            _p(router_w) if logits is None else 0, rows.shape[1] if logits is None else 0, stream_ptr())
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    mixers().grouped_router(logits.data_ptr(), _p(correction), T, E, int(count), int(keep), int(top), float(scale),
+                            ids.data_ptr(), wts.data_ptr(), stream_ptr())
     return ids, wts
 
 
