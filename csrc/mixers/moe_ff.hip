@@ -353,9 +353,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
 }
 
 // ---- prompt-sized steps (layout tiles of 64 or 128 rows): a workgroup owns 16 MT rows x 4 x 16 NT columns. The A rows
-// (gathered token rows, shared by the four waves) go through LDS, 32 k at a time in two buffers, one barrier
-// per step; every wave streams its own B columns from global memory into registers.
-template <int MODE, int MT, int NT>
+// (gathered token rows, shared by the four waves) go through LDS, KS = 32 or 64 k at a time in two buffers, one barrier
+// per step; every wave streams its own B columns from global memory into registers, with PF one step ahead of their
+// use (measured: 64-wide steps with the loads ahead gain about a tenth for one weight block per expert, and lose for the
+// gated form, whose two weight blocks per step then cost a third of the occupancy).
+template <int MODE, int MT, int NT, int KS, bool PF>
 __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* __restrict__ A, int64_t lda,
                                                                     const bf16* __restrict__ Wt,
                                                                     const int32_t* __restrict__ rows,
@@ -364,7 +366,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* 
                                                                     int kind, float limit, float alpha,
                                                                     const float* __restrict__ row_scale) {
   constexpr bool GATED = MODE == kGemmGated, FIRST = MODE != kGemmRows;
-  constexpr int LDA = 40, NG = GATED ? NT : 1, RPT = MT / 4;  // RPT: staged rows per thread
+  constexpr int LDA = KS + 8, NG = GATED ? NT : 1, RPT = MT / 4;  // RPT: staged rows per thread
+  constexpr int KH = KS / 32;                                     // 32-wide k halves (MFMA depth) per step
   __shared__ __attribute__((aligned(16))) uint16_t As[2][16 * MT * LDA];
   const int tile = blockIdx.x;  // 16 MT rows of a layout tile of tm rows
   const int e = tile_expert[tile * 16 * MT / tm];
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* 
   const int64_t wrows = GATED ? 2 * (int64_t)Nout : (int64_t)Nout;
   const bf16* We = Wt + (int64_t)e * wrows * K;
   const int rbase = tile * 16 * MT;
-  // staging: thread -> (rows tid / 4 + 64 r, 16-byte chunk = tid % 4) of the (16 MT) x 32 A block
+  // staging: thread -> (rows tid / 4 + 64 r, 16-byte chunks tid % 4 (+ 4)) of the (16 MT) x KS A block
   const int srow = threadIdx.x >> 2, sch = threadIdx.x & 3;
   int pa[RPT];
   const bf16* asrc[RPT];
@@ -392,38 +395,67 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_lds_kernel(const bf16* 
 #pragma unroll
     for (int j = 0; j < NG; ++j) accu[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
+  const bool wave_on = n0 < Nout;
+  // this wave's B rows (whole 16-column tiles; clamped ones are not stored)
+  const bf16* brow[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) brow[j] = We + (int64_t)(min(n0 + 16 * j, Nout - 16) + l16) * K + kg * 8;
+  uint4 bv[NT][KH], uv[NG][KH];
+  auto load_b = [&](int k0, uint4 (&b)[NT][KH], uint4 (&u)[NG][KH]) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int h = 0; h < KH; ++h) {
+        b[j][h] = ld16(brow[j] + k0 + 32 * h);
+        if (GATED) u[GATED ? j : 0][h] = ld16(brow[j] + (int64_t)Nout * K + k0 + 32 * h);
+      }
+  };
 #pragma unroll
   for (int r = 0; r < RPT; ++r)
-    xgk::st16(&As[0][(srow + 64 * r) * LDA + sch * 8], pa[r] >= 0 ? ld16(asrc[r]) : make_uint4(0, 0, 0, 0));
+#pragma unroll
+    for (int h = 0; h < KH; ++h)
+      xgk::st16(&As[0][(srow + 64 * r) * LDA + sch * 8 + 32 * h],
+                pa[r] >= 0 ? ld16(asrc[r] + 32 * h) : make_uint4(0, 0, 0, 0));
+  if (PF && wave_on) load_b(0, bv, uv);
   __syncthreads();
   int buf = 0;
-  const bool wave_on = n0 < Nout;
-  for (int k0 = 0; k0 < K; k0 += 32, buf ^= 1) {
-    const bool more = k0 + 32 < K;
-    uint4 anext[RPT];
+  for (int k0 = 0; k0 < K; k0 += KS, buf ^= 1) {
+    const bool more = k0 + KS < K;
+    uint4 anext[RPT][KH], bn[NT][KH], un[NG][KH];
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) anext[r] = (more && pa[r] >= 0) ? ld16(asrc[r] + k0 + 32) : make_uint4(0, 0, 0, 0);
+    for (int r = 0; r < RPT; ++r)
+#pragma unroll
+      for (int h = 0; h < KH; ++h)
+        anext[r][h] = (more && pa[r] >= 0) ? ld16(asrc[r] + k0 + KS + 32 * h) : make_uint4(0, 0, 0, 0);
     if (wave_on) {
-      uint4 bv[NT], uv[NG];
+      if (!PF) load_b(k0, bv, uv);
+      else if (more) load_b(k0 + KS, bn, un);
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const int n = min(n0 + 16 * j, Nout - 16) + l16;  // whole 16-column tiles; clamped ones are not stored
-        bv[j] = ld16(We + (int64_t)n * K + k0 + kg * 8);
-        if (GATED) uv[j] = ld16(We + (int64_t)(Nout + n) * K + k0 + kg * 8);
-      }
+      for (int h = 0; h < KH; ++h)
 #pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        const uint4 av = ld16(&As[buf][(16 * i + l16) * LDA + kg * 8]);
+        for (int i = 0; i < MT; ++i) {
+          const uint4 av = ld16(&As[buf][(16 * i + l16) * LDA + 32 * h + kg * 8]);
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          acc[i][j] = mfma16x16x32(as_frag(av), as_frag(bv[j]), acc[i][j]);
-          if (GATED) accu[i][j] = mfma16x16x32(as_frag(av), as_frag(uv[GATED ? j : 0]), accu[i][GATED ? j : 0]);
+          for (int j = 0; j < NT; ++j) {
+            acc[i][j] = mfma16x16x32(as_frag(av), as_frag(bv[j][h]), acc[i][j]);
+            if (GATED) accu[i][j] = mfma16x16x32(as_frag(av), as_frag(uv[GATED ? j : 0][h]), accu[i][GATED ? j : 0]);
+          }
         }
+      if (PF && more) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int h = 0; h < KH; ++h) {
+            bv[j][h] = bn[j][h];
+            if (GATED) uv[GATED ? j : 0][h] = un[GATED ? j : 0][h];
+          }
       }
     }
     if (more) {
 #pragma unroll
-      for (int r = 0; r < RPT; ++r) xgk::st16(&As[buf ^ 1][(srow + 64 * r) * LDA + sch * 8], anext[r]);
+      for (int r = 0; r < RPT; ++r)
+#pragma unroll
+        for (int h = 0; h < KH; ++h) xgk::st16(&As[buf ^ 1][(srow + 64 * r) * LDA + sch * 8 + 32 * h], anext[r][h]);
     }
     __syncthreads();
   }
@@ -496,9 +528,16 @@ int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int
 #define XGM_GG(MODE, K64)                                                                                           \
   grouped_gemm_mfma_kernel<MODE, 1, 2, true, K64><<<dim3(cap / tm, (Nout + 31) / 32), 256, 0, st>>>(                 \
       (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha, row_scale);
-#define XGM_GL(MODE, MT, NT)                                                                                          \
-  grouped_gemm_mfma_lds_kernel<MODE, MT, NT><<<dim3(cap / (16 * MT), (Nout + 64 * NT - 1) / (64 * NT)), 256, 0, st>>>( \
-      (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, tm, top, Nout, K, out, kind, limit, alpha, row_scale);
+#define XGM_GL2(MODE, MT, NT, KS, PF)                                                                                  \
+  grouped_gemm_mfma_lds_kernel<MODE, MT, NT, KS, PF>                                                                   \
+      <<<dim3(cap / (16 * MT), (Nout + 64 * NT - 1) / (64 * NT)), 256, 0, st>>>(                                       \
+          (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, tm, top, Nout, K, out, kind, limit, alpha, row_scale);
+#define XGM_GL(MODE, MT, NT)                 \
+  if (MODE != kGemmGated && K % 64 == 0) {   \
+    XGM_GL2(MODE, MT, NT, 64, true)          \
+  } else {                                   \
+    XGM_GL2(MODE, MT, NT, 32, false)         \
+  }
     if (tm == 128) {         // gated: 64 x 128 per workgroup (two accumulator sets); one weight block: 128 x 128
       if (mode == kGemmGated) { XGM_GL(kGemmGated, 4, 2) } else if (mode == kGemmAct) { XGM_GL(kGemmAct, 8, 2) } else { XGM_GL(kGemmRows, 8, 2) }
     } else if (tm == 64) {   // gated: 64 x 128; one weight block: 64 x 256
@@ -509,6 +548,7 @@ int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int
       if (mode == kGemmGated) { XGM_GG(kGemmGated, false) } else if (mode == kGemmAct) { XGM_GG(kGemmAct, false) } else { XGM_GG(kGemmRows, false) }
     }
 #undef XGM_GL
+#undef XGM_GL2
 #undef XGM_GG
     return 0;
   }
