@@ -7,7 +7,10 @@
 //                    split into `count` contiguous groups of equal size, a group is rated by the sum of its two
 //                    highest selection scores, members of the `keep` highest-rated groups stay eligible (all
 //                    others are excluded outright: selection score -inf); the `top` highest eligible selection
-//                    scores win; weight = score * scale (the correction does not enter it, no normalisation)
+//                    scores win; weight = score * scale (the correction does not enter it, no normalisation).
+//                    For steps of few rows the logits x . rw[e] (fp32 rows and router weights) are formed here
+//                    by a four-wave workgroup per token, eight experts per sweep over the row, instead of being
+//                    read (the waves then repeat the same selection, so every barrier is met by all of them).
 //   moe_align        (token, choice) pairs sorted by expert into tiles of `tm` rows (padded with -1)
 //   grouped_gemm     per tile: rows x expert weights, in one of three modes:
 //                      kGemmRows    A rows as they lie in the sorted layout -> fp32 rows (the second product)
@@ -58,22 +61,70 @@ __global__ void glu_act_kernel(const T* __restrict__ in, int64_t ld, T* __restri
 // ------------------------------------------------------------------ router: one wave per token
 constexpr int kMaxEPL = 8;  // experts per lane: E <= 512
 
-__global__ __launch_bounds__(64) void grouped_router_kernel(const float* __restrict__ logits, const float* __restrict__ corr,
-                                                            int E, int count, int keep, int top, float scale,
-                                                            int32_t* __restrict__ ids, float* __restrict__ wts) {
+constexpr int kRouterSweep = 8;   // experts per sweep over the row when the logits are formed here
+
+__global__ __launch_bounds__(256) void grouped_router_kernel(const float* __restrict__ logits, const float* __restrict__ corr,
+                                                             int E, int count, int keep, int top, float scale,
+                                                             int32_t* __restrict__ ids, float* __restrict__ wts,
+                                                             const float* __restrict__ x, const float* __restrict__ rw,
+                                                             int W) {
   extern __shared__ float sm[];
   float* cs = sm;              // [E] choice scores
   float* gs = sm + E;          // [count] group scores
   int* kept = (int*)(gs + count);  // [count]
-  const int t = blockIdx.x, lane = threadIdx.x;
+  float* lg = (float*)(kept + count);   // [E] logits formed here (x != nullptr)
+  float* part = lg + E;                 // [waves][kRouterSweep] partial sums
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int per = E / count;
+  if (x) {
+    const float* xr = x + (int64_t)t * W;
+    const bool vec = (W & 3) == 0;
+    for (int e0 = 0; e0 < E; e0 += kRouterSweep) {
+      float acc[kRouterSweep];
+#pragma unroll
+      for (int j = 0; j < kRouterSweep; ++j) acc[j] = 0.f;
+      if (vec) {
+        for (int c = 4 * threadIdx.x; c < W; c += 4 * blockDim.x) {
+          float a[4];
+          ld4(xr + c, a);
+#pragma unroll
+          for (int j = 0; j < kRouterSweep; ++j)
+            if (e0 + j < E) {
+              float b[4];
+              ld4(rw + (int64_t)(e0 + j) * W + c, b);
+              acc[j] += a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+            }
+        }
+      } else {
+        for (int c = threadIdx.x; c < W; c += blockDim.x) {
+          const float a = xr[c];
+#pragma unroll
+          for (int j = 0; j < kRouterSweep; ++j)
+            if (e0 + j < E) acc[j] += a * rw[(int64_t)(e0 + j) * W + c];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kRouterSweep; ++j) acc[j] = wave_sum(acc[j]);
+      if (lane == 0) {
+#pragma unroll
+        for (int j = 0; j < kRouterSweep; ++j) part[wave * kRouterSweep + j] = acc[j];
+      }
+      __syncthreads();
+      if (threadIdx.x < kRouterSweep && e0 + threadIdx.x < E) {
+        float v = 0.f;
+        for (int w = 0; w < nw; ++w) v += part[w * kRouterSweep + threadIdx.x];
+        lg[e0 + threadIdx.x] = v;
+      }
+      __syncthreads();
+    }
+  }
   float sc[kMaxEPL], ch[kMaxEPL];
 #pragma unroll
   for (int i = 0; i < kMaxEPL; ++i) {
     const int e = lane + 64 * i;
     sc[i] = 0.f, ch[i] = -INFINITY;
     if (e < E) {
-      sc[i] = sigmoidf(logits[(int64_t)t * E + e]);
+      sc[i] = sigmoidf(x ? lg[e] : logits[(int64_t)t * E + e]);
       ch[i] = sc[i] + (corr ? corr[e] : 0.f);
       cs[e] = ch[i];
     }
@@ -245,7 +296,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
                                                                 const float* __restrict__ row_scale) {
   constexpr bool GATED = MODE == kGemmGated, FIRST = MODE != kGemmRows;
   constexpr int NG = GATED ? NT : 1;
-  __shared__ float red[SPLITK ? 3 : 1][SPLITK ? (NT + NG) : 1][64][4];
+  __shared__ float red[SPLITK ? 3 : 1][SPLITK ? MT * (NT + NG) : 1][64][4];
   const int tile = blockIdx.x;          // layout tile of 16 MT rows
   const int e = tile_expert[tile];
   if (e < 0) return;
@@ -305,17 +356,20 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
           if (GATED) accu[i][j] = mfma16x16x32(as_frag(av[i][h]), as_frag(uv[j][h]), accu[i][j]);
         }
   }
-  if (SPLITK) {  // MT == 1: waves 1..3 hand their partial sums to wave 0
+  if (SPLITK) {  // waves 1..3 hand their partial sums to wave 0
     if (wave > 0) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int i = 0; i < MT; ++i) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[wave - 1][j][lane][r] = acc[0][j][r];
-      if (GATED) {
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
-        for (int j = 0; j < NG; ++j)
+          for (int r = 0; r < 4; ++r) red[wave - 1][i * (NT + NG) + j][lane][r] = acc[i][j][r];
+        if (GATED) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) red[wave - 1][NT + j][lane][r] = accu[0][j][r];
+          for (int j = 0; j < NG; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[wave - 1][i * (NT + NG) + NT + j][lane][r] = accu[i][j][r];
+        }
       }
     }
     __syncthreads();
@@ -323,14 +377,17 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(const bf16* __re
 #pragma unroll
     for (int w = 0; w < 3; ++w) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int i = 0; i < MT; ++i) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[0][j][r] += red[w][j][lane][r];
-      if (GATED) {
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
-        for (int j = 0; j < NG; ++j)
+          for (int r = 0; r < 4; ++r) acc[i][j][r] += red[w][i * (NT + NG) + j][lane][r];
+        if (GATED) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) accu[0][j][r] += red[w][NT + j][lane][r];
+          for (int j = 0; j < NG; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) accu[i][j][r] += red[w][i * (NT + NG) + NT + j][lane][r];
+        }
       }
     }
   }
@@ -499,12 +556,15 @@ void glu_act(const void* in, bool f32, int64_t ld, void* out, int T_, int F, int
 }
 
 int grouped_router(const float* logits, const float* corr, int T_, int E, int count, int keep, int top, float scale,
-                   int32_t* ids, float* wts, hipStream_t st) {
+                   int32_t* ids, float* wts, const float* x, const float* rw, int W, hipStream_t st) {
   if (T_ <= 0) return 0;
   if (E < 1 || E > 64 * kMaxEPL || count < 1 || E % count != 0 || keep < 1 || keep > count || top < 1 ||
       top > keep * (E / count))
     return -1;
-  grouped_router_kernel<<<T_, 64, (E + 2 * count) * sizeof(float), st>>>(logits, corr, E, count, keep, top, scale, ids, wts);
+  if ((x != nullptr) != (rw != nullptr) || (x && W < 1) || (!x && !logits)) return -2;
+  const int nth = x ? 256 : 64;
+  const size_t lds = (2 * E + 2 * count + 4 * kRouterSweep) * sizeof(float);
+  grouped_router_kernel<<<T_, nth, lds, st>>>(logits, corr, E, count, keep, top, scale, ids, wts, x, rw, W);
   return 0;
 }
 
@@ -520,14 +580,22 @@ int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int
                  int cap, int tm, int top, int Nout, int K, int mode, void* out, int kind, float limit, float alpha,
                  const float* row_scale, bool mfma, hipStream_t st) {
   if (cap <= 0) return 0;
-  if ((tm != 16 && tm != 64 && tm != 128) || cap % tm != 0 || Nout < 1 || K < 1 || mode < kGemmRows || mode > kGemmAct ||
+  if ((tm != 16 && tm != 32 && tm != 64 && tm != 128) || cap % tm != 0 || Nout < 1 || K < 1 || mode < kGemmRows || mode > kGemmAct ||
       (mode == kGemmGated && kind != kGluGeluTanh && kind != kGluClamped) || (mode == kGemmAct && kind != kActRelu2) ||
       (row_scale && mode != kGemmAct))
     return -1;
   if (!f32 && mfma && K % 32 == 0 && Nout % 16 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)Wt % 16 == 0) {
-#define XGM_GG(MODE, K64)                                                                                           \
-  grouped_gemm_mfma_kernel<MODE, 1, 2, true, K64><<<dim3(cap / tm, (Nout + 31) / 32), 256, 0, st>>>(                 \
+  // few rows per expert: layout tiles of 16 rows, or of 32 once many experts would fill more than one such tile (an
+  // expert's weights are then streamed once instead of once per 16 rows)
+#define XGM_GG2(MODE, MT, K64)                                                                                      \
+  grouped_gemm_mfma_kernel<MODE, MT, 2, true, K64><<<dim3(cap / tm, (Nout + 31) / 32), 256, 0, st>>>(                \
       (const bf16*)A, lda, (const bf16*)Wt, rows, tile_expert, top, Nout, K, out, kind, limit, alpha, row_scale);
+#define XGM_GG(MODE, K64)     \
+  if (tm == 32) {             \
+    XGM_GG2(MODE, 2, K64)     \
+  } else {                    \
+    XGM_GG2(MODE, 1, K64)     \
+  }
 #define XGM_GL2(MODE, MT, NT, KS, PF)                                                                                  \
   grouped_gemm_mfma_lds_kernel<MODE, MT, NT, KS, PF>                                                                   \
       <<<dim3(cap / (16 * MT), (Nout + 64 * NT - 1) / (64 * NT)), 256, 0, st>>>(                                       \
@@ -550,6 +618,7 @@ int grouped_gemm(const void* A, bool f32, int64_t lda, const void* Wt, const int
 #undef XGM_GL
 #undef XGM_GL2
 #undef XGM_GG
+#undef XGM_GG2
     return 0;
   }
   dim3 grid(cap / 16, (Nout + 63) / 64);

@@ -46,7 +46,8 @@ int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, con
 void gated_group_norm(const float*, const void*, bool, int64_t, const float*, int, float, void*, int, int, int, bool,
                       hipStream_t);
 void glu_act(const void*, bool, int64_t, void*, int, int, int, float, float, hipStream_t);
-int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, hipStream_t);
+int grouped_router(const float*, const float*, int, int, int, int, int, float, int32_t*, float*, const float*,
+                   const float*, int, hipStream_t);
 int moe_align(const int32_t*, int, int, int, int, int32_t*, int32_t*, int32_t*, hipStream_t);
 int grouped_gemm(const void*, bool, int64_t, const void*, const int32_t*, const int32_t*, int, int, int, int, int, int, void*,
                  int, float, float, const float*, bool, hipStream_t);
@@ -251,9 +252,9 @@ PYBIND11_MODULE(_mixers, m) {
     check(0, "glu_act");
   });
   m.def("grouped_router", [](uintptr_t logits, uintptr_t corr, int T, int E, int count, int keep, int top, float scale,
-                             uintptr_t ids, uintptr_t wts, uintptr_t st) {
+                             uintptr_t ids, uintptr_t wts, uintptr_t x, uintptr_t rw, int W, uintptr_t st) {
     int rc = xgm::grouped_router(P<const float>(logits), P<const float>(corr), T, E, count, keep, top, scale,
-                                 P<int32_t>(ids), P<float>(wts), S(st));
+                                 P<int32_t>(ids), P<float>(wts), P<const float>(x), P<const float>(rw), W, S(st));
     check(rc, "grouped_router");
   });
   m.def("moe_align", [](uintptr_t ids, int pairs, int E, int cap, int tm, uintptr_t rows, uintptr_t tile_expert,

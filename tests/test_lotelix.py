@@ -672,6 +672,11 @@ def test_experts_scaled_at_their_input(device, dtype, T, E, top, K, F_):
     down = torch.stack([w[f"e{e}.down"] for e in range(E)]).to(dt).to(device)
     got = sq.routed_experts(h.to(dt).to(device), up, down, ids, wts, sq.ACT_RELU2, scale_input=True)
     assert rel_err(got, ref) < (1e-4 if dtype == "float32" else 3e-2)
+    # the logits formed inside the router kernel (short steps) or by a matrix product (long ones)
+    ids2, wts2 = sq.grouped_router(None, None, 1, 1, top, 1.0, rows=h.float().to(device),
+                                   router_w=w["router"].float().to(device))
+    assert torch.equal(ids2.cpu().long().sort(-1).values, ids.cpu().long().sort(-1).values)
+    assert float((wts2.sort(-1).values - wts.sort(-1).values).abs().max()) < 1e-5
     # the sum over a token's choices inside the residual update
     rows = sq.routed_experts(h.to(dt).to(device), up, down, ids, wts, sq.ACT_RELU2, scale_input=True, combine=False)
     x = torch.randn(T, K, generator=g)

@@ -176,7 +176,7 @@ class InputScaledMoE(nn.Module):
 
     def forward(self, n32, nact):
         """The experts' output rows; the residual update sums them per token."""
-        ids, wts = sq.grouped_router(F.linear(n32, self.router), None, 1, 1, self.top, 1.0)
+        ids, wts = sq.grouped_router(None, None, 1, 1, self.top, 1.0, rows=n32, router_w=self.router)
         return sq.routed_experts(nact, self.up, self.down, ids, wts, sq.ACT_RELU2, scale_input=True, combine=False)
 
 

@@ -672,7 +672,9 @@ GLU_GELU_TANH, GLU_CLAMPED = 0, 1
 ACT_RELU2 = 2   # routed_experts(kind=...): an expert without a gate, W_down relu(W_up h)^2
 # XGS_TUNE moe_mfma=0: the general grouped GEMM for bf16 too (A/B and tests)
 MOE_MFMA = tune.get_bool("moe_mfma", True)
-MOE_TILE_SMALL, MOE_TILES_BIG = 16, (128, 64)   # rows per expert tile of the sorted layout
+MOE_TILE_SMALL, MOE_TILES_BIG = 16, (128, 64, 32)   # rows per expert tile of the sorted layout
+MOE_TILE32_MIN = 12   # average rows per expert from which 32-row tiles replace 16-row ones (XGS_TUNE moe_tile32_min)
+MOE_TILE32_MIN = tune.get_int("moe_tile32_min", MOE_TILE32_MIN)
 
 
 def _glu_ref(g, u, kind, limit, alpha):
@@ -698,15 +700,27 @@ def glu_act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.702
     return out
 
 
-def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], count: int, keep: int, top: int,
-                   scale: float):
-    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]). Scores are
+ROUTER_FUSED_MAX_ROWS = 256   # steps of up to this many rows form the router logits inside the router kernel
+
+
+def grouped_router(logits: Optional[torch.Tensor], correction: Optional[torch.Tensor], count: int, keep: int, top: int,
+                   scale: float, rows: Optional[torch.Tensor] = None, router_w: Optional[torch.Tensor] = None):
+    """fp32 router logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]). With `rows` (fp32 [T, W]) and
+    `router_w` (fp32 [E, W]) in place of `logits` the logits are rows . router_w[e] in fp32: inside the router kernel
+    for steps of few rows on the GPU (a launch less; the library product wins on long steps), else a matrix product. Scores are
     sigmoid(logits). Selection uses score + correction: the experts form `count` contiguous groups of equal
     size, a group is rated by the sum of its two highest selection scores, and only members of the `keep`
     highest-rated groups are eligible (everything else is excluded outright, selection score -inf). The
     returned weights are score * scale: the correction does not enter them and they are not normalised."""
-    T, E = logits.shape
-    if not native_device(logits):
+    fused = False
+    if logits is None:
+        assert rows.dtype == router_w.dtype == torch.float32 and rows.shape[1] == router_w.shape[1]
+        fused = native_device(rows) and rows.shape[0] <= ROUTER_FUSED_MAX_ROWS and rows.is_contiguous() \
+            and router_w.is_contiguous()
+        if not fused:
+            logits = torch.nn.functional.linear(rows, router_w)
+    T, E = (rows.shape[0], router_w.shape[0]) if fused else logits.shape
+    if not fused and not native_device(logits):
         s = torch.sigmoid(logits.float())
         c = s + (correction if correction is not None else 0.0)
         per = E // count
@@ -716,11 +730,13 @@ def grouped_router(logits: torch.Tensor, correction: Optional[torch.Tensor], cou
         c = c.masked_fill(~kept.repeat_interleave(per, 1), float("-inf"))
         ids = c.topk(top, -1).indices
         return ids.to(torch.int32), s.gather(1, ids) * scale
-    assert logits.dtype == torch.float32 and logits.is_contiguous()
-    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
-    wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    mixers().grouped_router(logits.data_ptr(), _p(correction), T, E, int(count), int(keep), int(top), float(scale),
-                            ids.data_ptr(), wts.data_ptr(), stream_ptr())
+    assert fused or (logits.dtype == torch.float32 and logits.is_contiguous())
+    dev = rows.device if fused else logits.device
+    ids = torch.empty(T, top, dtype=torch.int32, device=dev)
+    wts = torch.empty(T, top, dtype=torch.float32, device=dev)
+    mixers().grouped_router(0 if fused else logits.data_ptr(), _p(correction), T, E, int(count), int(keep), int(top),
+                            float(scale), ids.data_ptr(), wts.data_ptr(), rows.data_ptr() if fused else 0,
+                            router_w.data_ptr() if fused else 0, rows.shape[1] if fused else 0, stream_ptr())
     return ids, wts
 
 
@@ -771,8 +787,9 @@ def routed_experts(h: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, ids: to
     assert h.is_contiguous() and w13.is_contiguous() and w2.is_contiguous() and w13.dtype == w2.dtype == h.dtype
     assert wts.dtype == torch.float32 and wts.is_contiguous()
     pairs = T * top
-    # rows of an expert are padded to whole tiles: 128 / 64-row tiles once the average expert has that many, else 16
-    tm = next((t for t in MOE_TILES_BIG if pairs >= t * E), MOE_TILE_SMALL)
+    # rows of an expert are padded to whole tiles: 128 / 64-row tiles once the average expert has that many; 32-row
+    # tiles once many experts would need a second 16-row tile (their weights would be streamed twice); else 16
+    tm = next((t for t in MOE_TILES_BIG if pairs >= (t if t > 32 else MOE_TILE32_MIN) * E), MOE_TILE_SMALL)
     cap = (pairs + E * (tm - 1) + tm - 1) // tm * tm
     dev = h.device
     meta = torch.empty(cap + cap // tm + pairs, dtype=torch.int32, device=dev)
