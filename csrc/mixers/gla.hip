@@ -16,6 +16,13 @@
 // the next tile's global loads are issued before the current tile's steps and stored after them). Per token
 // a wave does 2 FMAs per owned state element; the waves' partial sums of o meet in LDS once per tile, in
 // wave order.
+//
+// Long portions, so that a few sequences still fill the chip: the recurrence is linear in S, so a chunk of kScanChunk
+// tokens is summed up by (A, B) with S_end = diag(A) S_start + B. A first launch (pass 1) runs every chunk from a
+// zero state without outputs and stores its A [dk] and B [dk x dv] (and sets the sequence's incoming state aside);
+// a second launch (pass 2) folds the chunks before its own onto the incoming state, in order, and runs its chunk
+// with outputs; the chunk that holds the last token writes the state back. Chunk slot of (sequence s, chunk z):
+// q0_s / kScanChunk + s + z, distinct for all chunks of a step and below T / kScanChunk + ns + 1.
 #include "mixers_common.h"
 
 namespace xgm {
@@ -56,13 +63,15 @@ __global__ void decay_gates_kernel(const T* __restrict__ proj, int64_t ld, int o
 // RAW: q and f are read as columns [off_q, off_q + H dk) / [off_f, ..) of the activation rows `raw` and go
 // through silu / the lower-bounded sigmoid while they are staged (no pass of their own, half the bytes), and the
 // write strength is 1 - f. Otherwise q, f (and k, or 1 - f when k == nullptr) are fp32 tensors [T, H dk].
+constexpr int kScanChunk = 256;
+
 template <typename T, int NI, int TT, int NW, bool RAW, int COLS>
 __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
     const float* __restrict__ q, const float* __restrict__ f, const float* __restrict__ k, const T* __restrict__ raw,
     int64_t ld_raw, int off_q, int off_f, const float* __restrict__ f_bias, const float* __restrict__ lower,
     const T* __restrict__ v, int64_t ld_v, float* __restrict__ state, const int32_t* __restrict__ qsl,
     const int32_t* __restrict__ seq_lens, const int32_t* __restrict__ slots, float* __restrict__ o, int H, int dk,
-    int dv) {
+    int dv, int pass, int nc, float* __restrict__ chA, float* __restrict__ chB, float* __restrict__ s_in) {
   constexpr int HALVES = 64 / COLS;          // row groups per wave
   constexpr int NB = NW * HALVES * NI;       // padded state rows
   constexpr int NTH = 64 * NW;
@@ -71,9 +80,12 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
   constexpr int PER = (TT * ROW + NTH - 1) / NTH;
   __shared__ __attribute__((aligned(16))) float stage[2][TT][ROW];
   __shared__ float opart[TT][NW][COLS];
-  const int s = blockIdx.x, h = blockIdx.y;
+  // pass 0: the whole portion in one workgroup; 1 / 2: chunk z of it (see above)
+  const int s = pass ? blockIdx.x / nc : blockIdx.x, z = pass ? blockIdx.x % nc : 0, h = blockIdx.y;
   const int q0 = qsl[s], qn = qsl[s + 1] - q0, slot = slots[s];
   if (slot < 0 || qn <= 0) return;
+  const int c0 = pass ? z * kScanChunk : 0, c1 = pass ? min(qn, c0 + kScanChunk) : qn;   // this workgroup's tokens
+  if (c0 >= qn) return;
   const int ctx = seq_lens[s] - qn;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane % COLS, rg = wave * HALVES + lane / COLS;   // column within the block, row group
@@ -81,15 +93,29 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
   const bool pok = p < dv;
   const int nqk = H * dk, nv = H * dv;
   float* Sg = state + (((int64_t)slot * H + h) * dk) * dv;
-  float S[NI];
+  float S[NI], Ap[NI];
+  const int64_t cs0 = pass ? q0 / kScanChunk + s : 0;   // the sequence's first chunk slot
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     const int n = rg * NI + i;
-    S[i] = (ctx > 0 && pok && n < dk) ? Sg[(int64_t)n * dv + p] : 0.f;
+    const bool ok = pok && n < dk;
+    Ap[i] = 1.f;
+    if (pass == 0) {
+      S[i] = (ctx > 0 && ok) ? Sg[(int64_t)n * dv + p] : 0.f;
+    } else if (pass == 1) {
+      if (z == 0 && ok) s_in[(((int64_t)s * H + h) * dk + n) * dv + p] = ctx > 0 ? Sg[(int64_t)n * dv + p] : 0.f;
+      S[i] = 0.f;
+    } else {
+      S[i] = ok ? s_in[(((int64_t)s * H + h) * dk + n) * dv + p] : 0.f;
+      for (int zc = 0; zc < z; ++zc) {
+        const int64_t cr = ((cs0 + zc) * H + h) * dk + n;
+        if (ok) S[i] = chA[cr] * S[i] + chB[cr * dv + p];
+      }
+    }
   }
   float pre[PER];
   auto fetch = [&](int t0) {  // global loads of the tile starting at token t0 (zeros past the end / the sizes)
-    const int nt = min(TT, qn - t0);
+    const int nt = min(TT, c1 - t0);
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int e = threadIdx.x + NTH * j;
@@ -138,13 +164,13 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
       }
     }
   };
-  fetch(0);
+  fetch(c0);
   commit(0);
   __syncthreads();
   int buf = 0;
-  for (int t0 = 0; t0 < qn; t0 += TT, buf ^= 1) {
-    const int nt = min(TT, qn - t0);
-    const bool more = t0 + TT < qn;
+  for (int t0 = c0; t0 < c1; t0 += TT, buf ^= 1) {
+    const int nt = min(TT, c1 - t0);
+    const bool more = t0 + TT < c1;
     if (more) fetch(t0 + TT);
     auto step = [&](int tt) {
       const float* fr = &stage[buf][tt][rg * NI];
@@ -158,6 +184,11 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
         S[i] = RAW ? fmaf(fr[i], S[i] - vv, vv) : fmaf(fr[i], S[i], kr[i] * vv);
         acc = fmaf(S[i], qr[i], acc);
       }
+      if (pass == 1) {   // the chunk's decay product; no outputs in this pass
+#pragma unroll
+        for (int i = 0; i < NI; ++i) Ap[i] *= fr[i];
+        return;
+      }
       if (HALVES == 2) acc += __shfl_xor(acc, 32, 64);
       if (lane < COLS) opart[tt][wave][col] = acc;
     };
@@ -168,7 +199,7 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
       for (int tt = 0; tt < nt; ++tt) step(tt);
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < nt * COLS; e += NTH) {
+    for (int e = threadIdx.x; pass != 1 && e < nt * COLS; e += NTH) {
       const int tt = e / COLS, c = e % COLS;
       if (p0 + c < dv) {
         float val = 0.f;
@@ -180,7 +211,17 @@ __global__ __launch_bounds__(64 * NW) void gated_linear_scan_kernel(
     if (more) commit(buf ^ 1);
     __syncthreads();
   }
-  if (pok) {
+  if (pass == 1) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = rg * NI + i;
+      const int64_t cr = ((cs0 + z) * H + h) * dk + n;
+      if (pok && n < dk) chB[cr * dv + p] = S[i];
+      if (p == 0 && n < dk) chA[cr] = Ap[i];
+    }
+    return;
+  }
+  if (pok && c1 == qn) {   // the workgroup that holds the last token
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int n = rg * NI + i;
@@ -206,21 +247,38 @@ void decay_gates(const void* proj, bool f32, int64_t ld, int off_q, int off_k, i
                           (const T*)proj, ld, off_q, off_k, n, q_scale, (const T*)z, ld_z, z_bias, inv_tau, q, f, k, total);)
 }
 
+int64_t gated_linear_scan_scratch_floats(int T_, int ns, int H, int dk, int dv) {
+  const int64_t cslots = T_ / kScanChunk + ns + 1;
+  return (cslots * (dv + 1) + (int64_t)ns * dv) * H * dk;
+}
+
 int gated_linear_scan(const float* q, const float* f, const float* k, const void* raw, int64_t ld_raw, int off_q, int off_f,
                       const float* f_bias, const float* lower, const void* v, bool v_f32, int64_t ld_v, float* state,
                       const int32_t* qsl, const int32_t* seq_lens, const int32_t* slots, float* o, int ns, int H, int dk,
-                      int dv, int cols_hint, hipStream_t st) {
+                      int dv, int cols_hint, float* scratch, int max_q, int T_, hipStream_t st) {
   if (ns <= 0) return 0;
   if (H <= 0 || dk < 1 || dk > 256 || dv < 1 || (raw ? !lower : (!q || !f))) return -1;
+  // long portions (scratch given): chunks of kScanChunk tokens over the whole grid, in two launches
+  const bool chunked = scratch && max_q > kScanChunk;
+  const int nc = chunked ? (max_q + kScanChunk - 1) / kScanChunk : 1;
+  const int64_t cslots = T_ / kScanChunk + ns + 1;
+  float* chA = scratch;
+  float* chB = chunked ? chA + cslots * H * dk : nullptr;
+  float* s_in = chunked ? chB + cslots * H * dk * dv : nullptr;
   // 32-column workgroups for small value sizes (no idle lanes), or on request. Doubling the workgroups of a step that
   // leaves compute units idle measured no faster: the scan is bound by the latency of a token step, not by lanes.
   const bool narrow = cols_hint == 32 || (cols_hint != 64 && dv <= 32);
   const int cols = narrow ? 32 : 64;
-  dim3 grid(ns, H, (dv + cols - 1) / cols);
-#define XGM_GL3(NI, TT, NW, RAW, COLS)                                                                                 \
-  XGM_DISPATCH_T(v_f32, gated_linear_scan_kernel<T, NI, TT, NW, RAW, COLS><<<grid, 64 * NW, 0, st>>>(                   \
-                            q, f, k, (const T*)raw, ld_raw, off_q, off_f, f_bias, lower, (const T*)v, ld_v, state, qsl, \
-                            seq_lens, slots, o, H, dk, dv);)
+  dim3 grid(ns * nc, H, (dv + cols - 1) / cols);
+#define XGM_GL4(NI, TT, NW, RAW, COLS, PASS)                                                                           \
+  gated_linear_scan_kernel<T, NI, TT, NW, RAW, COLS><<<grid, 64 * NW, 0, st>>>(                                         \
+      q, f, k, (const T*)raw, ld_raw, off_q, off_f, f_bias, lower, (const T*)v, ld_v, state, qsl, seq_lens, slots, o, H, \
+      dk, dv, PASS, nc, chA, chB, s_in);
+#define XGM_GL3(NI, TT, NW, RAW, COLS)                                               \
+  XGM_DISPATCH_T(v_f32, if (chunked) {                                               \
+    XGM_GL4(NI, TT, NW, RAW, COLS, 1)                                                \
+    XGM_GL4(NI, TT, NW, RAW, COLS, 2)                                                \
+  } else { XGM_GL4(NI, TT, NW, RAW, COLS, 0) })
   // NI rows per lane: the narrow form covers twice the rows per wave, so it takes half of them per lane
 #define XGM_GL2(NI, TT, NW, RAW)          \
   if (narrow) {                           \
@@ -244,6 +302,7 @@ int gated_linear_scan(const float* q, const float* f, const float* k, const void
 #undef XGM_GL
 #undef XGM_GL2
 #undef XGM_GL3
+#undef XGM_GL4
 }
 
 }  // namespace xgm

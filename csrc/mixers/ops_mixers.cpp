@@ -40,7 +40,8 @@ void lower_bound_gates(const void*, bool, int64_t, int, int, int, const float*, 
                        hipStream_t);
 int gated_linear_scan(const float*, const float*, const float*, const void*, int64_t, int, int, const float*, const float*,
                       const void*, bool, int64_t, float*, const int32_t*, const int32_t*, const int32_t*, float*, int, int,
-                      int, int, int, hipStream_t);
+                      int, int, int, float*, int, int, hipStream_t);
+int64_t gated_linear_scan_scratch_floats(int, int, int, int, int);
 int ssm_scan(const void*, bool, int64_t, const void*, int64_t, const float*, const float*, const float*, float*,
              const int32_t*, const int32_t*, const int32_t*, float*, int, int, int, int, int, hipStream_t);
 void gated_group_norm(const float*, const void*, bool, int64_t, const float*, int, float, void*, int, int, int, bool,
@@ -217,16 +218,19 @@ PYBIND11_MODULE(_mixers, m) {
   m.def("gated_linear_scan", [](uintptr_t q, uintptr_t f, uintptr_t k, uintptr_t raw, int64_t ld_raw, int off_q, int off_f,
                                 uintptr_t f_bias, uintptr_t lower, uintptr_t v, bool v_f32, int64_t ld_v, uintptr_t state,
                                 uintptr_t qsl, uintptr_t sl, uintptr_t slots, uintptr_t o, int ns, int H, int dk, int dv,
-                                int cols_hint, uintptr_t st) {
+                                int cols_hint, uintptr_t scratch, int max_q, int T, uintptr_t st) {
     if (H < 1 || dv < 1 || dk < 1 || ld_v < (int64_t)H * dv ||
         (raw && (off_q < 0 || off_f < 0 || ld_raw < off_q + (int64_t)H * dk || ld_raw < off_f + (int64_t)H * dk)))
       throw std::invalid_argument("gated_linear_scan: inconsistent sizes");
     int rc = xgm::gated_linear_scan(P<const float>(q), P<const float>(f), P<const float>(k), P<const void>(raw), ld_raw,
                                     off_q, off_f, P<const float>(f_bias), P<const float>(lower), P<const void>(v), v_f32,
                                     ld_v, P<float>(state), P<const int32_t>(qsl), P<const int32_t>(sl),
-                                    P<const int32_t>(slots), P<float>(o), ns, H, dk, dv, cols_hint, S(st));
+                                    P<const int32_t>(slots), P<float>(o), ns, H, dk, dv, cols_hint, P<float>(scratch),
+                                    max_q, T, S(st));
     check(rc, "gated_linear_scan");
   });
+  m.def("gated_linear_scan_scratch_floats",
+        [](int T, int ns, int H, int dk, int dv) { return xgm::gated_linear_scan_scratch_floats(T, ns, H, dk, dv); });
   m.def("ssm_scan", [](uintptr_t xbc, bool f32, int64_t ld_x, uintptr_t dt, int64_t ld_dt, uintptr_t dt_bias,
                        uintptr_t A_log, uintptr_t D, uintptr_t state, uintptr_t qsl, uintptr_t sl, uintptr_t slots,
                        uintptr_t y, int ns, int H, int G, int N, int Pd, uintptr_t st) {

@@ -613,14 +613,20 @@ def test_sink_can_take_all_the_weight(device):
 
 @pytest.mark.parametrize("device", OP_CASES)
 @pytest.mark.parametrize("H,dk,dv,tau,rank", [(3, 20, 12, 5.0, 6), (2, 16, 16, 1.0, 1), (1, 6, 70, 16.0, 3), (2, 64, 80, 2.5, 8)])
-def test_decayed_linear_attention_over_portions_and_slots(device, H, dk, dv, tau, rank):
+@pytest.mark.parametrize("lens,cuts", [((29, 11), [[5, 1, 1, 2, 17, 1, 2], [2, 2, 1, 1, 5]]),
+                                       ((900, 40), [[3, 600, 1, 257, 39], [20, 1, 2, 1, 16]])], ids=["short", "long"])
+@pytest.mark.parametrize("two_pass", [True, False], ids=["chunks", "one-workgroup"])
+def test_decayed_linear_attention_over_portions_and_slots(device, H, dk, dv, tau, rank, lens, cuts, two_pass, monkeypatch):
+    """Short portions and single tokens, and portions of several hundred tokens (scanned as chunks over the whole grid,
+    in two launches, beside another sequence's short portions), on slots with leftovers."""
+    monkeypatch.setattr(sq, "SCAN_TWO_PASS", two_pass)
     g = torch.Generator().manual_seed(dk)
     W, eps = 24, 1e-5
     m = {"heads": H, "dim": dk, "vdim": dv, "tau": tau, "decay_rank": rank}
     cfg = {"width": W, "vocab": 8, "layers": [{"type": "parallel", "mlp": None, "mixer": {
         "left": {"heads": 1, "kv_heads": 1, "dim": 4, "vdim": 4, "scale": 1.0}, "right": m}}]}
     Wt = {k[len("l0.mix.right."):]: v for k, v in orc.random_weights(cfg, seed=dk).items() if k.startswith("l0.mix.right.")}
-    hs = [torch.randn(n, W, generator=g).to(F64) for n in (29, 11)]
+    hs = [torch.randn(n, W, generator=g).to(F64) for n in lens]
     refs = [orc.decayed_linear_attention(h, Wt, "", m, eps) for h in hs]
     n, nv = H * dk, H * dv
     Wcat = torch.cat([Wt["q"], Wt["k"], Wt["v"], Wt["g"], Wt["a1"]])
@@ -634,7 +640,7 @@ def test_decayed_linear_attention_over_portions_and_slots(device, H, dk, dv, tau
         o = sq.gated_linear_scan(q, fg, k, proj[:, 2 * n:2 * n + nv], state, H, dk, dv, sm)
         y = sq.gated_group_norm(o, proj[:, 2 * n + nv:2 * n + 2 * nv], f(Wt["norm"]), eps, H, torch.float32, gate_after=True)
         return (y.cpu().to(F64) @ Wt["o"].T).float()
-    got = in_portions(device, hs, [[5, 1, 1, 2, 17, 1, 2], [2, 2, 1, 1, 5]], [1, 2], fn)
+    got = in_portions(device, hs, cuts, [1, 2], fn)
     for a, b in zip(got, refs):
         assert rel_err(a, b) < 1e-4
 

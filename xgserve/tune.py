@@ -38,7 +38,7 @@ from typing import Dict
 
 KEYS = {"fused_decode", "async_sched", "early_release", "spin_wait", "pf", "pf_windows", "moe_pf", "moe_w2_small", "argmax_split", "gemm_ar", "gemm_ar_shared", "small_m_tiles", "krot", "m64_plans", "mw_plans",
         "mw_max_tokens", "resid_inlaunch_kb", "decode_depth", "decode_max_splits", "ar_ll_max", "sim_ar_us",
-        "tp_overlap_chunks", "tp_overlap_min_tokens", "ep_exact_min_pairs", "latent_mfma", "delta_two_pass", "attn_mfma", "attn_waves", "scan_cols", "conv_prep_fused", "moe_mfma", "mingru_two_pass", "moe_tile32_min"}
+        "tp_overlap_chunks", "tp_overlap_min_tokens", "ep_exact_min_pairs", "latent_mfma", "delta_two_pass", "attn_mfma", "attn_waves", "scan_cols", "conv_prep_fused", "moe_mfma", "mingru_two_pass", "moe_tile32_min", "scan_two_pass"}
 
 
 def _parse(spec: str) -> Dict[str, str]:
