@@ -539,7 +539,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(
     const float* __restrict__ wk, float eps, const float* __restrict__ rot, int rot_rows, int rot_dims,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_mapping, TO* __restrict__ q_out,
     TO* __restrict__ kcache, TO* __restrict__ vcache, int whole, int half, const TI* __restrict__ v_first,
-    int64_t ld_vf, const float* __restrict__ v_mix) {
+    int64_t ld_vf, const float* __restrict__ v_mix, int vec) {
   __shared__ float red[4];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -568,6 +568,67 @@ __global__ __launch_bounds__(256) void head_norm_rope_cache_kernel(
     }
   }
   const int hr = rot_dims / 2;
+  if (vec) {
+    // four consecutive entries per thread (no per-head statistic to wait for): a pair lies inside the quad
+    // (2i, 2i + 1) or in the quad rot_dims / 2 further on / back (i, i + rot_dims / 2)
+    const int qpd = dk / 4;   // quads per head
+    for (int e = threadIdx.x; e < (H + G) * qpd; e += blockDim.x) {
+      const int hd = e / qpd, d0 = 4 * (e % qpd);
+      const bool is_q = hd < H;
+      if (!is_q && slot < 0) continue;
+      const int hh = is_q ? hd : hd - H;
+      const TI* v = row + (is_q ? hd * dk : nq + hh * dk);
+      const float* w = is_q ? wq : wk;
+      const float* wh = w ? w + hh * dk : nullptr;   // whole-vector weights
+      const float r = is_q ? rq : rk;
+      float a[4], g[4] = {1.f, 1.f, 1.f, 1.f};
+      ld4(v + d0, a);
+      if (wh) ld4(wh + d0, g);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] *= r * g[i];
+      if (cs && d0 < rot_dims) {
+        if (half) {
+          const bool second = d0 >= hr;
+          const int pd0 = second ? d0 - hr : d0 + hr, pi = second ? d0 - hr : d0;
+          float b[4], cs0[4], cs1[4];
+          ld4(v + pd0, b);
+          if (wh) ld4(wh + pd0, g);
+          ld4(cs + 2 * pi, cs0);        // (c, s) of pairs pi, pi + 1
+          ld4(cs + 2 * pi + 4, cs1);    // ... pi + 2, pi + 3
+          const float c[4] = {cs0[0], cs0[2], cs1[0], cs1[2]}, sn[4] = {cs0[1], cs0[3], cs1[1], cs1[3]};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float bb = b[i] * r * g[i];
+            a[i] = second ? a[i] * c[i] + bb * sn[i] : a[i] * c[i] - bb * sn[i];
+          }
+        } else {
+          float cq[4];
+          ld4(cs + d0, cq);             // (c, s) of pairs d0 / 2, d0 / 2 + 1
+          const float u0 = a[0], v0 = a[1], u1 = a[2], v1 = a[3];
+          a[0] = u0 * cq[0] - v0 * cq[1];
+          a[1] = v0 * cq[0] + u0 * cq[1];
+          a[2] = u1 * cq[2] - v1 * cq[3];
+          a[3] = v1 * cq[2] + u1 * cq[3];
+        }
+      }
+      st4((is_q ? q_out + (int64_t)t * nq + hd * dk : kcache + (int64_t)slot * nk + hh * dk) + d0, a);
+    }
+    if (slot >= 0) {
+      const float lam = v_first ? *v_mix : 0.f;
+      for (int c = 4 * threadIdx.x; c < nv; c += 4 * blockDim.x) {
+        float a[4];
+        ld4(row + nq + nk + c, a);
+        if (v_first) {
+          float b[4];
+          ld4(v_first + (int64_t)t * ld_vf + c, b);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a[i] = (1.f - lam) * a[i] + lam * b[i];
+        }
+        st4(vcache + (int64_t)slot * nv + c, a);
+      }
+    }
+    return;
+  }
   for (int hd = wave; hd < H + G; hd += nw) {
     const bool is_q = hd < H;
     if (!is_q && slot < 0) continue;   // padding row: nothing is cached
@@ -835,11 +896,21 @@ void head_norm_rope_cache(const void* src, bool src_f32, int64_t ld, int H, int 
                           bool out_f32, int T_, bool whole, bool half, const void* v_first, int64_t ld_vf,
                           const float* v_mix, hipStream_t st) {
   if (T_ <= 0) return;
+  // four entries per thread where no per-head statistic is needed (no norm, or norms over the whole vectors) and
+  // quads stay whole: head sizes, value rows and strides multiples of 4, rotated pairs inside a quad (2i, 2i + 1) or
+  // a whole number of quads apart (i, i + n / 2), rows aligned to 16 (float) / 8 (bf16) bytes
+  const int isz = src_f32 ? 4 : 2, osz = out_f32 ? 4 : 2;
+  const bool use_rot = rot && rot_dims > 0;
+  const int vec = ((!wq && !wk) || whole) && dk % 4 == 0 && (G * dv) % 4 == 0 && ld % 4 == 0 &&
+                  (uintptr_t)src % (4 * isz) == 0 && (uintptr_t)q_out % (4 * osz) == 0 &&
+                  (uintptr_t)kcache % (4 * osz) == 0 && (uintptr_t)vcache % (4 * osz) == 0 &&
+                  (!use_rot || (half ? rot_dims % 8 == 0 : rot_dims % 4 == 0)) &&
+                  (!v_first || (ld_vf % 4 == 0 && (uintptr_t)v_first % (4 * isz) == 0));
 #define XGM_HN(TI, TO)                                                                                               \
   head_norm_rope_cache_kernel<TI, TO><<<T_, 256, 0, st>>>((const TI*)src, ld, H, G, dk, dv, wq, wk, eps, rot, rot_rows, \
                                                           rot_dims, positions, slot_mapping, (TO*)q_out, (TO*)kcache,  \
                                                           (TO*)vcache, whole ? 1 : 0, half ? 1 : 0, (const TI*)v_first, \
-                                                          ld_vf, v_mix);
+                                                          ld_vf, v_mix, vec);
   if (src_f32) {
     if (out_f32) { XGM_HN(float, float) } else { XGM_HN(float, bf16) }
   } else {

@@ -17,7 +17,7 @@
 
 namespace xgm {
 
-constexpr int kMaxNormGroups = 64;
+constexpr int kMaxNormGroups = 256;
 
 template <typename TY, typename TO>
 __global__ __launch_bounds__(256) void residual_norm_kernel(float* __restrict__ x, const TY* __restrict__ y1, int64_t ld1,

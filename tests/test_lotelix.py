@@ -402,7 +402,7 @@ def in_portions(device, xs, cuts, slots, fn, tables=None, block_size=4):
 
 
 @pytest.mark.parametrize("device", OP_CASES)
-@pytest.mark.parametrize("W,groups", [(77, 1), (77, 7), (96, 2), (96, 8), (90, 3), (2304, 2), (2304, 64)])
+@pytest.mark.parametrize("W,groups", [(77, 1), (77, 7), (96, 2), (96, 8), (90, 3), (2304, 2), (2304, 64), (1024, 256)])
 def test_residual_sum_and_group_norm(device, W, groups):
     """x + y, x + fp32 sum, and the mean of two branches that are each normed first; the norm in `groups` parts, also
     with parts that are no multiple of four columns."""

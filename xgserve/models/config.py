@@ -336,8 +336,8 @@ def lotelix_config(name: str, width: int, vocab: int, layers: List[dict], embed_
                 need(rot["scaling"], ("factor", "low", "high", "original"), w)
     if not layers:
         raise ValueError("a model needs at least one layer")
-    if norm_groups < 1 or norm_groups > 64 or width % norm_groups:
-        raise ValueError("norm.groups must be in [1, 64] and divide the width")
+    if norm_groups < 1 or norm_groups > 256 or width % norm_groups:
+        raise ValueError("norm.groups must be in [1, 256] and divide the width")
     mixed = None
     for i, L in enumerate(layers):
         m, w = L.get("mixer") or {}, f"layer {i}"
