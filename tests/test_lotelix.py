@@ -655,10 +655,10 @@ def test_decay_of_a_very_negative_logit_stays_finite(device):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("T,E,top,K,F_", [(7, 5, 2, 40, 24), (50, 1, 1, 32, 16), (300, 3, 3, 64, 48), (700, 4, 1, 96, 64),
+@pytest.mark.parametrize("T,E,top,K,F_", [(7, 5, 2, 40, 24), (50, 1, 1, 32, 16), (100, 1, 1, 64, 32), (300, 3, 3, 64, 48), (700, 4, 1, 96, 64),
                                           (1300, 4, 2, 128, 32), (64, 12, 1, 24, 10)])
 def test_experts_scaled_at_their_input(device, dtype, T, E, top, K, F_):
-    """Every grouped-GEMM path (tiles of 16, 64 and 128 rows; matrix-core and general) against the dense form in which
+    """Every grouped-GEMM path (tiles of 16, 32, 64 and 128 rows; matrix-core and general) against the dense form in which
     the routing score multiplies the expert's input; scores far from one, so a weight applied at the output (which the
     squared activation would turn into its square) shows."""
     dt = getattr(torch, dtype)
